@@ -1,0 +1,173 @@
+/*
+ * tccl_amd.h -- C ABI of the MI355X (gfx950) data path for tccl-style collectives.
+ *
+ * One GPU holds W "virtual ranks": W separate device allocations stand in for the
+ * symmetric-memory peer buffers of the reference.  Every entry point below replaces one
+ * Triton kernel launch (or one host helper) of the reference; the file:line each one
+ * replaces is given with it (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - plain C: pointers and sizes only, no torch types.
+ *   - every device pointer must be 16-byte aligned; `stream` is a hipStream_t passed as
+ *     void* (NULL = the null stream).
+ *   - calls are asynchronous on `stream`, allocate nothing, never synchronise and never
+ *     throw; the return value is TCCL_OK or a negative code (tccl_error_string()).
+ *   - ordering between virtual ranks and between tree levels is stream order; this
+ *     replaces the reference's signal-pad barrier (triton_barrier.py:39-142) and its
+ *     wait/send flags (triton_double_tree_allreduce.py:175-225).
+ *   - float sums: each bf16 is widened to fp32, accumulated from +0.0f in the order the
+ *     sources are given, and rounded once (round-to-nearest-even) on store.  NaN sign
+ *     and payload are not specified.
+ */
+#ifndef TCCL_AMD_H
+#define TCCL_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TCCL_ABI_VERSION 1
+
+/* Largest number of source buffers one launch can take (virtual world size). */
+#define TCCL_MAX_WORLD 8
+/* Largest number of node steps one tccl_tree_level() launch can take. */
+#define TCCL_MAX_JOBS 8
+/* Largest world the host-side tree index math accepts. */
+#define TCCL_MAX_TREE_WORLD (1 << 20)
+
+enum {
+    TCCL_OK = 0,
+    TCCL_EINVAL = -1,      /* NULL pointer, world/rank/dtype out of range, size mismatch */
+    TCCL_EALIGN = -2,      /* a pointer or a row size is not a multiple of 16 bytes */
+    TCCL_EPOW2 = -3,       /* tree world size is not a power of two >= 2 */
+    TCCL_EHIP_BASE = -1000 /* -(1000 + hipError_t) */
+};
+
+typedef enum {
+    TCCL_BF16 = 0, /* bf16 in/out, fp32 accumulate, one RNE rounding */
+    TCCL_F32 = 1   /* fp32 in/out, fp32 accumulate */
+} tccl_dtype_t;
+
+/* Launch shape override, for tuning and tests.  Any field left 0 is chosen by the
+ * library.  The reference hard-codes its shape in each wrapper
+ * (triton_one_shot_all_reduce_no_128.py:68-71: 24 blocks x 512 lanes). */
+typedef struct {
+    int block;      /* threads per workgroup: 64, 128, 256 or 512 */
+    int unroll;     /* independent 16-byte vectors per thread per iteration: 1, 2 or 4 */
+    int grid;       /* workgroups (per source row for the gather) */
+    int tile_iters; /* consecutive iterations a workgroup spends on one contiguous tile */
+    int flags;      /* TCCL_CFG_* */
+} tccl_launch_cfg;
+
+#define TCCL_CFG_NONTEMPORAL_LOAD 1  /* mark loads as streaming */
+#define TCCL_CFG_NONTEMPORAL_STORE 2 /* mark stores as streaming */
+#define TCCL_CFG_XCD_CONTIGUOUS 4    /* give each of the 8 XCDs one contiguous eighth of the tiles */
+#define TCCL_CFG_TEMPORAL 8          /* force plain (cached) loads and stores */
+
+int tccl_abi_version(void);
+const char *tccl_error_string(int code);
+
+/* One-shot all-reduce (sum): out[j] = sum_{i<world} bufs[i][j].
+ * Replaces one_shot_all_reduce_kernel, triton_one_shot_all_reduce_no_128.py:35-64
+ * (launched at :85-95).  `bufs` is a HOST array of `world` device pointers (the
+ * reference's symm_mem.buffer_ptrs_dev, :86, passed here by value into the kernel
+ * arguments).  1 <= world <= TCCL_MAX_WORLD.  `numel` may be any value; elements past
+ * the last whole 16-byte vector are summed one at a time. */
+int tccl_all_reduce_sum(const void *const *bufs, int world, void *out, size_t numel,
+                        int dtype, void *stream);
+int tccl_all_reduce_sum_ex(const void *const *bufs, int world, void *out, size_t numel,
+                           int dtype, void *stream, const tccl_launch_cfg *cfg);
+
+/* One rank's share of a reduce-scatter: out[j] = sum_i bufs[i][rank*P + j],
+ * P = numel_total / world, j < P.
+ * Replaces one_shot_reduce_scatter_kernel, triton_reduce_scatter.py:59-92 (launched at
+ * :116-126).  rank*P*esize must be a multiple of 16 (the reference requires
+ * numel % (8*world) == 0, :101-104). */
+int tccl_reduce_scatter_sum(const void *const *bufs, int world, int rank, void *out,
+                            size_t numel_total, int dtype, void *stream);
+int tccl_reduce_scatter_sum_ex(const void *const *bufs, int world, int rank, void *out,
+                               size_t numel_total, int dtype, void *stream,
+                               const tccl_launch_cfg *cfg);
+
+/* All-gather pack: out is [world, bytes_per_rank] row-major, row i = bufs[i].
+ * Replaces one_shot_all_gather_kernel, triton_all_gather.py:32-63 (launched at :84-94;
+ * output layout :82).  Typeless byte copy; bytes_per_rank % 16 == 0. */
+int tccl_all_gather(const void *const *bufs, int world, void *out, size_t bytes_per_rank,
+                    void *stream);
+int tccl_all_gather_ex(const void *const *bufs, int world, void *out, size_t bytes_per_rank,
+                       void *stream, const tccl_launch_cfg *cfg);
+
+/* Double-tree node step, reduce half: dst[j] = 0 + child0[j] + child1[j] + own[j] in that
+ * order; a NULL child is skipped (the reference's -1).  dst may be `own` (the reference
+ * stores in place, triton_double_tree_allreduce.py:293-294).
+ * Replaces the reduce loop of double_tree_all_reduce_kernel,
+ * triton_double_tree_allreduce.py:266-295 including the child adds at :276-288. */
+int tccl_tree_reduce_step(const void *own, const void *child0, const void *child1, void *dst,
+                          size_t numel, int dtype, void *stream);
+
+/* Double-tree node step, forward/broadcast half: dst0[j] = dst1[j] = src[j]; dst1 may be
+ * NULL.  Replaces the broadcast loop sketched at
+ * triton_double_tree_allreduce.py:306-326 (own <- parent, output <- parent).
+ * bytes % 16 == 0. */
+int tccl_tree_copy_step(const void *src, void *dst0, void *dst1, size_t bytes, void *stream);
+
+/* A batch of independent node steps in ONE launch (all nodes of one tree level, both
+ * trees).  No counterpart in the reference, where each rank's kernel does its own step;
+ * on one GPU the steps of a level are independent and share a launch. */
+typedef struct {
+    const void *src[3]; /* reduce: child0, child1, own (NULL = absent); copy: src[0] only */
+    void *dst[2];       /* dst[1] may be NULL */
+    size_t numel;       /* elements of `dtype` */
+    int is_copy;        /* 0 = reduce step, 1 = copy step (bit-exact, no arithmetic) */
+    int pad_;
+} tccl_node_job;
+
+int tccl_tree_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_elems,
+                    void *stream);
+
+/* Tree index math (host only, no GPU needed).
+ * tccl_double_tree_arrays  replaces build_double_tree, tree.py:34-91 (heap-ordered arrays).
+ * tccl_double_tree_indices replaces get_parents_and_children, tree.py:93-148:
+ *   out6 = (a_parent, a_child0, a_child1, b_parent, b_child0, b_child1), -1 = none.
+ * world must be a power of two >= 2 (tree.py:11; world == 1 fails in the reference at
+ * tree.py:135). */
+int tccl_double_tree_arrays(int world, int *tree_a, int *tree_b);
+int tccl_double_tree_indices(int world, int rank, int *out6);
+
+/* First element of the half that tree b reduces: floor(numel/2) rounded down to whole
+ * 16-byte vectors.  Tree a owns [0, split), tree b owns [split, numel). */
+size_t tccl_double_tree_split(size_t numel, size_t esize);
+
+/* The whole double-tree all-reduce for all `world` virtual ranks, as the sequence of node
+ * steps that triton_double_tree_allreduce.py:254-335 (live and commented code) describes,
+ * one launch per tree level with both trees in it, ordered by the stream:
+ * up-sweep  -- each interior node reduces its children's buffers into its own, in place;
+ * down-sweep -- each rank copies its parent's buffer into its own buffer and its output.
+ * bufs[r] is overwritten with the result (as in the reference's design, :293-294 and
+ * :321-323); outs[r] (nullable entries) receive rank r's output (:324-325).  `world` is a
+ * power of two, 2..TCCL_MAX_WORLD.  chunk_elems = elements per pipelining chunk
+ * (0 = 128 KiB worth). */
+int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs, int world, size_t numel,
+                                int dtype, size_t chunk_elems, void *stream);
+
+/* HIP-event helpers so a host language without HIP bindings can time launches on the very
+ * stream they run on.  No counterpart in the reference (it times with torch.cuda.Event,
+ * triton_reduce_scatter.py:216-226). */
+int tccl_event_create(void **event_out);
+int tccl_event_destroy(void *event);
+int tccl_event_record(void *event, void *stream);
+int tccl_event_synchronize(void *event);
+int tccl_event_elapsed_ms(void *start, void *stop, float *ms_out);
+int tccl_stream_synchronize(void *stream);
+
+/* Device facts used for reporting: compute units, memory clock (kHz), bus width (bits),
+ * L2 bytes.  Any pointer may be NULL. */
+int tccl_device_info(int *compute_units, int *mem_clock_khz, int *mem_bus_bits, size_t *l2_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TCCL_AMD_H */

@@ -1,0 +1,67 @@
+"""Build recipe for ``libtccl_amd.so`` (hipcc, gfx950 only).
+
+``python -m tccl_amd.build`` compiles every ``csrc/*.hip`` into an object file and links
+the shared library next to this file.  The library is built in-tree so that it travels
+with the source tree; nothing is compiled at import time.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+from typing import List
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(CSRC, "_obj")
+LIB_PATH = os.path.join(HERE, "libtccl_amd.so")
+
+SOURCES = ["sum.hip", "gather.hip", "tree.hip", "util.hip"]
+
+# -ffp-contract=off: the sums are adds only, but nothing may ever be fused.
+# -packed-fp32-ops off: keep the compiler from forming v_pk_add_f32 out of the
+# accumulator adds; each add stays a scalar v_add_f32.
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; libtccl_amd.so can only be built with ROCm's hipcc")
+    return exe
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
+    return obj
+
+
+def build(verbose: bool = False, jobs: int = 4) -> str:
+    """Compile and link the library; returns its path.  Always recompiles."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs: List[str] = list(pool.map(_compile, SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH)} bytes)")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build(verbose=True)
+    sys.exit(0)

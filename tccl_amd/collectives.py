@@ -1,0 +1,147 @@
+"""The four collectives with the reference's call signatures, for virtual ranks on one GPU.
+
+Each function takes *this rank's* buffer, finds its peers with ``rendezvous`` exactly as
+the reference's wrappers do, allocates the output with torch and launches one HIP kernel
+(one per tree level for the double tree) through the C ABI on torch's current stream.
+Preconditions are the reference's own assertions, raised before anything is launched.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+from .symm import SymmGroup, SymmHandle, rendezvous
+
+_SUM_DTYPES = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _sum_dtype(tensor: torch.Tensor) -> int:
+    # the reference takes bfloat16 only (triton_one_shot_all_reduce_no_128.py:73); float32
+    # is summed with the same kernel and no final rounding
+    assert tensor.dtype in _SUM_DTYPES, "Only bfloat16 (and float32) is supported for now."
+    return _SUM_DTYPES[tensor.dtype]
+
+
+def _vec_elems(tensor: torch.Tensor) -> int:
+    return 16 // tensor.element_size()
+
+
+def _cfg_ptr(cfg: Optional[_lib.LaunchCfg]):
+    return ctypes.byref(cfg) if cfg is not None else None
+
+
+def one_shot_all_reduce(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
+    """Sum of all ranks' buffers over ``tensor.numel()`` elements.
+
+    Mirrors ``one_shot_all_reduce`` (triton_one_shot_all_reduce_no_128.py:67-96): same
+    dtype and alignment assertions (:73-76), a fresh ``empty_like`` output (:83).  The sum
+    is accumulated in fp32 in rank order and rounded once."""
+    dtype = _sum_dtype(tensor)
+    assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
+    symm = rendezvous(tensor)
+    output = torch.empty_like(tensor)
+    lib = _lib.load()
+    rc = lib.tccl_all_reduce_sum_ex(symm.buffer_ptrs_host, symm.world_size, output.data_ptr(), tensor.numel(),
+                                    dtype, _stream(), _cfg_ptr(cfg))
+    _lib.check("tccl_all_reduce_sum", rc)
+    return output
+
+
+def one_shot_reduce_scatter(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
+    """This rank's 1/W share of the sum: elements ``[rank*P, (rank+1)*P)``, ``P = numel // W``.
+
+    Mirrors ``one_shot_reduce_scatter`` (triton_reduce_scatter.py:95-127); rank and world
+    size come from the handle (the reference reads module globals, :103-113)."""
+    dtype = _sum_dtype(tensor)
+    symm = rendezvous(tensor)
+    world, rank = symm.world_size, symm.rank
+    assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
+    per_rank = tensor.numel() // world
+    flat = tensor.reshape(-1)
+    output = torch.empty_like(flat[per_rank * rank:per_rank * (rank + 1)])
+    lib = _lib.load()
+    rc = lib.tccl_reduce_scatter_sum_ex(symm.buffer_ptrs_host, world, rank, output.data_ptr(), tensor.numel(),
+                                        dtype, _stream(), _cfg_ptr(cfg))
+    _lib.check("tccl_reduce_scatter_sum", rc)
+    return output
+
+
+def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, *,
+                        cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
+    """``[W, *tensor.shape]`` tensor whose row i is a copy of rank i's buffer.
+
+    Mirrors ``one_shot_all_gather(tensor, world_size)`` (triton_all_gather.py:66-95).  Any
+    dtype is copied bit for bit (the reference asserts bfloat16, :72, though its copy is
+    typeless); the byte count per rank must be a multiple of 16 (:73-75)."""
+    symm = rendezvous(tensor)
+    if world_size is None:
+        world_size = symm.world_size
+    assert world_size == symm.world_size, "world_size does not match the tensor's symmetric group"
+    nbytes = tensor.numel() * tensor.element_size()
+    assert nbytes % 16 == 0, "The number of elements must be 128-bit aligned."
+    output = torch.empty((world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
+    lib = _lib.load()
+    rc = lib.tccl_all_gather_ex(symm.buffer_ptrs_host, world_size, output.data_ptr(), nbytes, _stream(),
+                                _cfg_ptr(cfg))
+    _lib.check("tccl_all_gather", rc)
+    return output
+
+
+def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tensor,
+                     chunk_elems: int) -> List[torch.Tensor]:
+    outputs = [torch.empty_like(like) for _ in range(group.world_size)]
+    lib = _lib.load()
+    out_ptrs = _lib.ptr_array([int(o.data_ptr()) for o in outputs])
+    rc = lib.tccl_double_tree_all_reduce(group.ptr_array, out_ptrs, group.world_size, numel, dtype, chunk_elems,
+                                         _stream())
+    _lib.check("tccl_double_tree_all_reduce", rc)
+    return outputs
+
+
+def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0) -> torch.Tensor:
+    """All-reduce over two complementary binary trees, one per half of the elements.
+
+    Mirrors ``double_tree_all_reduce`` (triton_double_tree_allreduce.py:338-370) as its
+    kernel was designed (:254-335): every interior node sums its children's buffers into
+    its own buffer in place, then every rank copies its parent's buffer into its own buffer
+    and its output.  World size and rank come from the handle (the reference hard-codes 8
+    and a global, :356).
+
+    A collective is one call per rank.  On one GPU the first rank to call runs the node
+    steps of *all* virtual ranks (the ranks' buffers are overwritten with the result, as
+    in the reference's design) and gets its output; the other ranks' outputs wait in the
+    group until those ranks call.  A rank calling again starts the next collective."""
+    dtype = _sum_dtype(tensor)
+    assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
+    symm = rendezvous(tensor)
+    group = symm.group
+    pending = group.pending_outputs.pop(symm.rank, None)
+    if pending is not None and pending.shape == tensor.shape:
+        return pending
+    outputs = _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems)
+    group.pending_outputs = {r: o for r, o in enumerate(outputs) if r != symm.rank}
+    return outputs[symm.rank]
+
+
+def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *,
+                                 chunk_elems: int = 0) -> List[torch.Tensor]:
+    """One whole collective for every virtual rank of ``group``; returns the W outputs."""
+    like = group.tensors[0].reshape(-1)
+    if numel is not None:
+        like = like[:numel]
+    dtype = _sum_dtype(like)
+    assert like.numel() % _vec_elems(like) == 0, "The number of elements must be 128-bit aligned."
+    group.pending_outputs.clear()
+    return _run_double_tree(group, like.numel(), dtype, like, chunk_elems)
+
+
+# BASELINE names for the same functions
+reduce_scatter = one_shot_reduce_scatter
+all_gather = one_shot_all_gather

@@ -1,0 +1,148 @@
+// sum.hip -- one-shot all-reduce, reduce-scatter share and the single tree reduce step:
+// all three are "sum NSRC source streams into one destination stream", launched over
+// pointers that the host passes by value in the kernel arguments (they live in SGPRs;
+// the reference re-reads a device pointer table for every rank in every iteration,
+// triton_one_shot_all_reduce_no_128.py:59).
+#include "host.h"
+#include "vec.h"
+
+namespace tccl {
+
+template <int NSRC>
+struct SrcTable {
+    const char *p[NSRC];
+};
+
+template <class Sum, int NSRC, int UNROLL, bool NTL, bool NTS>
+__global__ void __launch_bounds__(kMaxBlock)
+sum_kernel(SrcTable<NSRC> src, char *out, size_t numel, int tile_iters, int xcd_contiguous)
+{
+    char *const dst[1] = {out};
+    sum_range<Sum, NSRC, 1, UNROLL, NTL, NTS>(src.p, dst, numel, tile_iters, xcd_contiguous != 0);
+}
+
+template <class Sum, int NSRC, int UNROLL, bool NTL, bool NTS>
+static hipError_t launch_sum(const char *const *srcs, char *out, size_t numel, const Shape &sh, hipStream_t stream)
+{
+    SrcTable<NSRC> t;
+    for (int i = 0; i < NSRC; ++i) t.p[i] = srcs[i];
+    hipLaunchKernelGGL((sum_kernel<Sum, NSRC, UNROLL, NTL, NTS>), dim3(sh.grid), dim3(sh.block), 0, stream, t, out,
+                       numel, sh.tile_iters, sh.xcd_contiguous ? 1 : 0);
+    return hipGetLastError();
+}
+
+template <class Sum, int NSRC, int UNROLL>
+static hipError_t launch_sum_nt(const char *const *srcs, char *out, size_t numel, const Shape &sh, hipStream_t stream)
+{
+    if (sh.nt_load) {
+        if (sh.nt_store) return launch_sum<Sum, NSRC, UNROLL, true, true>(srcs, out, numel, sh, stream);
+        return launch_sum<Sum, NSRC, UNROLL, true, false>(srcs, out, numel, sh, stream);
+    }
+    if (sh.nt_store) return launch_sum<Sum, NSRC, UNROLL, false, true>(srcs, out, numel, sh, stream);
+    return launch_sum<Sum, NSRC, UNROLL, false, false>(srcs, out, numel, sh, stream);
+}
+
+template <class Sum, int NSRC>
+static hipError_t launch_sum_unroll(const char *const *srcs, char *out, size_t numel, const Shape &sh,
+                                    hipStream_t stream)
+{
+    switch (sh.unroll) {
+    case 1: return launch_sum_nt<Sum, NSRC, 1>(srcs, out, numel, sh, stream);
+    case 2: return launch_sum_nt<Sum, NSRC, 2>(srcs, out, numel, sh, stream);
+    default:
+        // 4 vectors x 8 sources would hold 128 data registers per lane; cap it at 2 there.
+        if constexpr (NSRC <= 4)
+            return launch_sum_nt<Sum, NSRC, 4>(srcs, out, numel, sh, stream);
+        else
+            return launch_sum_nt<Sum, NSRC, 2>(srcs, out, numel, sh, stream);
+    }
+}
+
+template <class Sum>
+static hipError_t launch_sum_nsrc(const char *const *srcs, int nsrc, char *out, size_t numel, const Shape &sh,
+                                  hipStream_t stream)
+{
+    switch (nsrc) {
+    case 1: return launch_sum_unroll<Sum, 1>(srcs, out, numel, sh, stream);
+    case 2: return launch_sum_unroll<Sum, 2>(srcs, out, numel, sh, stream);
+    case 3: return launch_sum_unroll<Sum, 3>(srcs, out, numel, sh, stream);
+    case 4: return launch_sum_unroll<Sum, 4>(srcs, out, numel, sh, stream);
+    case 5: return launch_sum_unroll<Sum, 5>(srcs, out, numel, sh, stream);
+    case 6: return launch_sum_unroll<Sum, 6>(srcs, out, numel, sh, stream);
+    case 7: return launch_sum_unroll<Sum, 7>(srcs, out, numel, sh, stream);
+    case 8: return launch_sum_unroll<Sum, 8>(srcs, out, numel, sh, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// Sum `nsrc` already-offset source pointers into `out`.  Shared by the three entry points.
+int sum_streams(const void *const *srcs, int nsrc, void *out, size_t numel, int dtype, hipStream_t stream,
+                const tccl_launch_cfg *cfg)
+{
+    const int esize = dtype_size(dtype);
+    if (esize == 0 || nsrc < 1 || nsrc > TCCL_MAX_WORLD || srcs == nullptr || out == nullptr) return TCCL_EINVAL;
+    for (int i = 0; i < nsrc; ++i) {
+        if (srcs[i] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(srcs[i])) return TCCL_EALIGN;
+    }
+    if (!aligned16(out)) return TCCL_EALIGN;
+    if (numel == 0) return TCCL_OK;
+
+    const size_t nvec = numel * static_cast<size_t>(esize) / kVecBytes;
+    const Shape sh = resolve_shape(cfg, nvec, nsrc, 1);
+    const char *const *s = reinterpret_cast<const char *const *>(srcs);
+    hipError_t e = (dtype == TCCL_BF16) ? launch_sum_nsrc<Bf16Sum>(s, nsrc, static_cast<char *>(out), numel, sh, stream)
+                                        : launch_sum_nsrc<F32Sum>(s, nsrc, static_cast<char *>(out), numel, sh, stream);
+    return hip_code(e);
+}
+
+} // namespace tccl
+
+using namespace tccl;
+
+extern "C" int tccl_all_reduce_sum_ex(const void *const *bufs, int world, void *out, size_t numel, int dtype,
+                                      void *stream, const tccl_launch_cfg *cfg)
+{
+    return sum_streams(bufs, world, out, numel, dtype, static_cast<hipStream_t>(stream), cfg);
+}
+
+extern "C" int tccl_all_reduce_sum(const void *const *bufs, int world, void *out, size_t numel, int dtype,
+                                   void *stream)
+{
+    return tccl_all_reduce_sum_ex(bufs, world, out, numel, dtype, stream, nullptr);
+}
+
+extern "C" int tccl_reduce_scatter_sum_ex(const void *const *bufs, int world, int rank, void *out,
+                                          size_t numel_total, int dtype, void *stream, const tccl_launch_cfg *cfg)
+{
+    const int esize = dtype_size(dtype);
+    if (esize == 0 || bufs == nullptr || world < 1 || world > TCCL_MAX_WORLD || rank < 0 || rank >= world)
+        return TCCL_EINVAL;
+    const size_t per_rank = numel_total / static_cast<size_t>(world);
+    const size_t byte_off = static_cast<size_t>(rank) * per_rank * static_cast<size_t>(esize);
+    if (byte_off % kVecBytes != 0) return TCCL_EALIGN;
+    const void *shifted[TCCL_MAX_WORLD];
+    for (int i = 0; i < world; ++i) {
+        if (bufs[i] == nullptr) return TCCL_EINVAL;
+        shifted[i] = static_cast<const char *>(bufs[i]) + byte_off;
+    }
+    return sum_streams(shifted, world, out, per_rank, dtype, static_cast<hipStream_t>(stream), cfg);
+}
+
+extern "C" int tccl_reduce_scatter_sum(const void *const *bufs, int world, int rank, void *out, size_t numel_total,
+                                       int dtype, void *stream)
+{
+    return tccl_reduce_scatter_sum_ex(bufs, world, rank, out, numel_total, dtype, stream, nullptr);
+}
+
+extern "C" int tccl_tree_reduce_step(const void *own, const void *child0, const void *child1, void *dst,
+                                     size_t numel, int dtype, void *stream)
+{
+    if (own == nullptr || dst == nullptr) return TCCL_EINVAL;
+    const void *srcs[3];
+    int n = 0;
+    if (child0) srcs[n++] = child0;
+    if (child1) srcs[n++] = child1;
+    srcs[n++] = own;
+    return sum_streams(srcs, n, dst, numel, dtype, static_cast<hipStream_t>(stream), nullptr);
+}

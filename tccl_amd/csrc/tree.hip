@@ -1,0 +1,300 @@
+// tree.hip -- the double binary tree: a batch of node steps per launch, and the schedule
+// that runs the whole collective for all virtual ranks as one launch per tree level.
+#include <vector>
+
+#include "host.h"
+#include "vec.h"
+
+namespace tccl {
+
+struct JobTable {
+    tccl_node_job job[TCCL_MAX_JOBS];
+};
+
+// One node step over its element range.  blockIdx.y selects the job; the workgroups of a
+// job walk its range one pipelining chunk (tile) at a time, so a chunk is read, reduced
+// and written by a single workgroup, the way one message of the tree pipeline would be.
+template <class Sum, int NSRC, int NDST>
+__device__ __forceinline__ void run_reduce(const tccl_node_job &j, const char *const (&src)[NSRC], int tile_iters)
+{
+    if constexpr (NDST == 2) {
+        char *const dst[2] = {static_cast<char *>(j.dst[0]), static_cast<char *>(j.dst[1])};
+        sum_range<Sum, NSRC, 2, 2, false, false>(src, dst, j.numel, tile_iters, false);
+    } else {
+        char *const dst[1] = {static_cast<char *>(j.dst[0])};
+        sum_range<Sum, NSRC, 1, 2, false, false>(src, dst, j.numel, tile_iters, false);
+    }
+}
+
+template <class Sum, int NDST>
+__device__ __forceinline__ void run_job(const tccl_node_job &j, int tile_iters)
+{
+    const char *c0 = static_cast<const char *>(j.src[0]);
+    const char *c1 = static_cast<const char *>(j.src[1]);
+    const char *own = static_cast<const char *>(j.src[2]);
+    if (j.is_copy) {
+        const size_t nvec = j.numel * Sum::kElemBytes / kVecBytes;
+        if constexpr (NDST == 2) {
+            char *const dst[2] = {static_cast<char *>(j.dst[0]), static_cast<char *>(j.dst[1])};
+            copy_range<2, 2, false, false>(c0, dst, nvec, tile_iters, false);
+        } else {
+            char *const dst[1] = {static_cast<char *>(j.dst[0])};
+            copy_range<1, 2, false, false>(c0, dst, nvec, tile_iters, false);
+        }
+    } else if (c0 != nullptr && c1 != nullptr) {
+        const char *const src[3] = {c0, c1, own};
+        run_reduce<Sum, 3, NDST>(j, src, tile_iters);
+    } else if (c0 != nullptr) {
+        const char *const src[2] = {c0, own};
+        run_reduce<Sum, 2, NDST>(j, src, tile_iters);
+    } else if (c1 != nullptr) {
+        const char *const src[2] = {c1, own};
+        run_reduce<Sum, 2, NDST>(j, src, tile_iters);
+    } else {
+        const char *const src[1] = {own};
+        run_reduce<Sum, 1, NDST>(j, src, tile_iters);
+    }
+}
+
+template <class Sum>
+__global__ void __launch_bounds__(kMaxBlock) tree_level_kernel(JobTable jobs, int tile_iters)
+{
+    const tccl_node_job &j = jobs.job[blockIdx.y];
+    if (j.dst[1] != nullptr)
+        run_job<Sum, 2>(j, tile_iters);
+    else
+        run_job<Sum, 1>(j, tile_iters);
+}
+
+constexpr int kLevelBlock = 256;
+constexpr int kLevelUnroll = 2; // matches the UNROLL used in run_reduce / run_job
+
+int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_elems, hipStream_t stream)
+{
+    const int esize = dtype_size(dtype);
+    if (esize == 0 || jobs == nullptr || njobs < 0 || njobs > TCCL_MAX_JOBS) return TCCL_EINVAL;
+    if (njobs == 0) return TCCL_OK;
+    const size_t per_vec = kVecBytes / esize;
+    if (chunk_elems == 0) chunk_elems = (128u * 1024u) / esize;
+    const size_t span = static_cast<size_t>(kLevelBlock) * kLevelUnroll; // vectors per iteration
+    size_t tile_iters = (chunk_elems / per_vec + span - 1) / span;
+    if (tile_iters < 1) tile_iters = 1;
+    if (tile_iters > (1u << 20)) return TCCL_EINVAL;
+
+    JobTable t = {};
+    size_t max_tiles = 0;
+    for (int i = 0; i < njobs; ++i) {
+        const tccl_node_job &j = jobs[i];
+        if (j.dst[0] == nullptr) return TCCL_EINVAL;
+        if (j.is_copy ? (j.src[0] == nullptr) : (j.src[2] == nullptr)) return TCCL_EINVAL;
+        for (int k = 0; k < 3; ++k)
+            if (!aligned16(j.src[k])) return TCCL_EALIGN;
+        if (!aligned16(j.dst[0]) || !aligned16(j.dst[1])) return TCCL_EALIGN;
+        if (j.is_copy && (j.numel % per_vec) != 0) return TCCL_EALIGN;
+        t.job[i] = j;
+        const size_t nvec = j.numel / per_vec;
+        const size_t tiles = (nvec + span * tile_iters - 1) / (span * tile_iters);
+        if (tiles > max_tiles) max_tiles = tiles;
+    }
+    if (max_tiles == 0) max_tiles = 1; // ragged tails only
+    // Enough workgroups over all jobs to fill the chip about eight deep, no more than one
+    // per chunk.
+    size_t want = (static_cast<size_t>(compute_units()) * 8 + njobs - 1) / njobs;
+    const unsigned gx = static_cast<unsigned>(max_tiles < want ? max_tiles : want);
+    if (dtype == TCCL_BF16)
+        hipLaunchKernelGGL(tree_level_kernel<Bf16Sum>, dim3(gx, njobs), dim3(kLevelBlock), 0, stream, t,
+                           static_cast<int>(tile_iters));
+    else
+        hipLaunchKernelGGL(tree_level_kernel<F32Sum>, dim3(gx, njobs), dim3(kLevelBlock), 0, stream, t,
+                           static_cast<int>(tile_iters));
+    return hip_code(hipGetLastError());
+}
+
+} // namespace tccl
+
+using namespace tccl;
+
+extern "C" int tccl_tree_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_elems, void *stream)
+{
+    return launch_level(jobs, njobs, dtype, chunk_elems, static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------------------------------ tree index math
+// Closed form of the heap-ordered array that tree.py:5-31 builds row by row: position
+// idx >= 1 sits on level L = floor(log2 idx) at column c = idx - 2^L, and holds the
+// in-order label (2c + 1) * world / 2^(L+1); position 0 holds the extra node 0.
+
+static bool pow2_world(int world) { return world >= 2 && world <= TCCL_MAX_TREE_WORLD && (world & (world - 1)) == 0; }
+
+extern "C" int tccl_double_tree_arrays(int world, int *tree_a, int *tree_b)
+{
+    if (!pow2_world(world)) return TCCL_EPOW2;
+    if (tree_a == nullptr || tree_b == nullptr) return TCCL_EINVAL;
+    tree_a[0] = 0;
+    for (int level_first = 1; level_first < world; level_first *= 2)
+        for (int c = 0; c < level_first; ++c)
+            tree_a[level_first + c] = (2 * c + 1) * (world / (2 * level_first));
+    // tree.py:83-91: the second tree is the first with every label lowered by one, the
+    // subroot wrapping round to world-1.
+    for (int i = 0; i < world; ++i) tree_b[i] = (tree_a[i] + world - 1) % world;
+    return TCCL_OK;
+}
+
+// Neighbours of `r` in tree a without building the array (tree.py:130-146 looks the rank
+// up in the array).  For r >= 1 let t = number of trailing zero bits: the node sits t
+// levels above the leaves, its children are r -/+ 2^(t-1), and its parent is r - 2^t when
+// bit t+1 of r is set, r + 2^t otherwise; the top interior node world/2 hangs under the
+// extra node 0, whose single child it is (tree.py:133-136).
+static void tree_a_neighbours(int world, int r, int *out3)
+{
+    if (r == 0) {
+        out3[0] = -1;
+        out3[1] = world / 2;
+        out3[2] = -1;
+        return;
+    }
+    const int low = r & -r;
+    if (r == world / 2)
+        out3[0] = 0;
+    else
+        out3[0] = (r & (low << 1)) ? r - low : r + low;
+    if (low == 1) {
+        out3[1] = -1;
+        out3[2] = -1;
+    } else {
+        out3[1] = r - low / 2;
+        out3[2] = r + low / 2;
+    }
+}
+
+extern "C" int tccl_double_tree_indices(int world, int rank, int *out6)
+{
+    if (!pow2_world(world)) return TCCL_EPOW2;
+    if (out6 == nullptr || rank < 0 || rank >= world) return TCCL_EINVAL;
+    tree_a_neighbours(world, rank, out6);
+    // Rank r plays in tree b the part that rank r+1 (mod world) plays in tree a; its
+    // neighbours are that node's neighbours lowered by one, mod world.  -1 stays -1.
+    tree_a_neighbours(world, (rank + 1) % world, out6 + 3);
+    for (int k = 3; k < 6; ++k)
+        if (out6[k] >= 0) out6[k] = (out6[k] + world - 1) % world;
+    return TCCL_OK;
+}
+
+extern "C" size_t tccl_double_tree_split(size_t numel, size_t esize)
+{
+    if (esize == 0 || esize > kVecBytes) return 0;
+    const size_t per_vec = kVecBytes / esize;
+    return (numel / 2) / per_vec * per_vec;
+}
+
+// ------------------------------------------------------------------ the whole collective
+// Levels of one tree, by height above the leaves: a rank r >= 1 of tree a is at height
+// ctz(r); the extra node 0 sits above the top interior node.  The up-sweep runs heights
+// 1 .. log2(world)-1 and then the extra node; leaves run no step of their own: their step
+// is "own <- 0 + own", which changes nothing a parent can see (the parent's accumulator
+// also starts at +0) and nothing the caller can see (the down-sweep overwrites the leaf's
+// buffer).  The down-sweep runs the same levels top to bottom, every rank pulling from its
+// parent.
+
+extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs, int world, size_t numel, int dtype,
+                                           size_t chunk_elems, void *stream)
+{
+    const int esize = dtype_size(dtype);
+    if (esize == 0 || bufs == nullptr) return TCCL_EINVAL;
+    if (!pow2_world(world)) return TCCL_EPOW2;
+    if (world > TCCL_MAX_WORLD) return TCCL_EINVAL;
+    for (int r = 0; r < world; ++r) {
+        if (bufs[r] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(bufs[r]) || (outs && !aligned16(outs[r]))) return TCCL_EALIGN;
+    }
+    const size_t per_vec = kVecBytes / esize;
+    if (numel % per_vec != 0) return TCCL_EALIGN;
+    if (numel == 0) return TCCL_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    const size_t split = tccl_double_tree_split(numel, esize);
+    const size_t lo[2] = {0, split};
+    const size_t len[2] = {split, numel - split};
+
+    int height = 0;
+    while ((1 << height) < world) ++height;
+
+    // node_height[tree][rank]: 0 = leaf, 1..height-1 = interior, height = the extra node.
+    int nbr[2][TCCL_MAX_WORLD][3];
+    int node_height[2][TCCL_MAX_WORLD];
+    for (int r = 0; r < world; ++r) {
+        int six[6];
+        int rc = tccl_double_tree_indices(world, r, six);
+        if (rc != TCCL_OK) return rc;
+        for (int t = 0; t < 2; ++t) {
+            for (int k = 0; k < 3; ++k) nbr[t][r][k] = six[3 * t + k];
+            const int ra = (t == 0) ? r : (r + 1) % world;
+            node_height[t][r] = (ra == 0) ? height : __builtin_ctz(ra);
+        }
+    }
+
+    auto at = [&](int rank, int tree) { return static_cast<char *>(bufs[rank]) + lo[tree] * esize; };
+    auto out_at = [&](int rank, int tree) -> char * {
+        return (outs && outs[rank]) ? static_cast<char *>(outs[rank]) + lo[tree] * esize : nullptr;
+    };
+
+    std::vector<tccl_node_job> batch;
+    auto flush = [&]() -> int {
+        for (size_t i = 0; i < batch.size(); i += TCCL_MAX_JOBS) {
+            const int n = static_cast<int>(batch.size() - i < TCCL_MAX_JOBS ? batch.size() - i : TCCL_MAX_JOBS);
+            int rc = launch_level(batch.data() + i, n, dtype, chunk_elems, s);
+            if (rc != TCCL_OK) return rc;
+        }
+        batch.clear();
+        return TCCL_OK;
+    };
+
+    // Up-sweep.
+    for (int h = 1; h <= height; ++h) {
+        for (int t = 0; t < 2; ++t) {
+            if (len[t] == 0) continue;
+            for (int r = 0; r < world; ++r) {
+                if (node_height[t][r] != h) continue;
+                tccl_node_job j = {};
+                const int c0 = nbr[t][r][1], c1 = nbr[t][r][2];
+                j.src[0] = c0 >= 0 ? at(c0, t) : nullptr;
+                j.src[1] = c1 >= 0 ? at(c1, t) : nullptr;
+                j.src[2] = at(r, t);
+                j.dst[0] = at(r, t);
+                j.dst[1] = nullptr;
+                j.numel = len[t];
+                j.is_copy = 0;
+                batch.push_back(j);
+            }
+        }
+        int rc = flush();
+        if (rc != TCCL_OK) return rc;
+    }
+
+    // Down-sweep: the extra node already holds the result; it only has to fill its output.
+    // Every other rank copies its parent's buffer into its own buffer and its output.
+    for (int h = height; h >= 0; --h) {
+        for (int t = 0; t < 2; ++t) {
+            if (len[t] == 0) continue;
+            for (int r = 0; r < world; ++r) {
+                if (node_height[t][r] != h) continue;
+                tccl_node_job j = {};
+                j.is_copy = 1;
+                j.numel = len[t];
+                if (h == height) {
+                    if (out_at(r, t) == nullptr) continue;
+                    j.src[0] = at(r, t);
+                    j.dst[0] = out_at(r, t);
+                } else {
+                    j.src[0] = at(nbr[t][r][0], t);
+                    j.dst[0] = at(r, t);
+                    j.dst[1] = out_at(r, t);
+                }
+                batch.push_back(j);
+            }
+        }
+        int rc = flush();
+        if (rc != TCCL_OK) return rc;
+    }
+    return TCCL_OK;
+}

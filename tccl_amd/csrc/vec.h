@@ -1,0 +1,259 @@
+// vec.h -- 16-byte vector access and the bf16/fp32 sum arithmetic shared by every kernel.
+//
+// Everything here is written for gfx950 wave64: one lane moves one 16-byte vector per
+// access (global_load_dwordx4 / global_store_dwordx4), so a wave instruction covers one
+// contiguous KiB.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace tccl {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kVecBytes = 16;
+constexpr int kMaxBlock = 512;
+constexpr int kNumXcd = 8;
+
+template <bool NT>
+__device__ __forceinline__ u32x4 load_vec(const char *base, size_t vec_index)
+{
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(base) + vec_index;
+    if constexpr (NT)
+        return __builtin_nontemporal_load(p);
+    else
+        return *p;
+}
+
+template <bool NT>
+__device__ __forceinline__ void store_vec(char *base, size_t vec_index, u32x4 v)
+{
+    u32x4 *p = reinterpret_cast<u32x4 *>(base) + vec_index;
+    if constexpr (NT)
+        __builtin_nontemporal_store(v, p);
+    else
+        *p = v;
+}
+
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Two fp32 -> two bf16 packed in a dword (element 0 in the low half), round to nearest
+// even: one v_cvt_pk_bf16_f32.
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
+{
+    f32x2 f = {lo, hi};
+    bf16x2 b = __builtin_convertvector(f, bf16x2);
+    return __builtin_bit_cast(uint32_t, b);
+}
+
+// bf16 sums: eight fp32 accumulators per 16-byte vector.
+struct Bf16Sum {
+    static constexpr int kElemBytes = 2;
+    float a[8];
+
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a[k] = 0.0f;
+    }
+    // Widening bf16 -> fp32 is a 16-bit shift (exact).
+    __device__ __forceinline__ void add(u32x4 v)
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            a[2 * k] = a[2 * k] + bits_to_f32(v[k] << 16);
+            a[2 * k + 1] = a[2 * k + 1] + bits_to_f32(v[k] & 0xFFFF0000u);
+        }
+    }
+    __device__ __forceinline__ u32x4 result() const
+    {
+        u32x4 r;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) r[k] = pack_bf16(a[2 * k], a[2 * k + 1]);
+        return r;
+    }
+    // One element at a time, for the ragged tail.
+    static __device__ __forceinline__ float widen(const char *p, size_t i)
+    {
+        return bits_to_f32(static_cast<uint32_t>(reinterpret_cast<const uint16_t *>(p)[i]) << 16);
+    }
+    static __device__ __forceinline__ void narrow(char *p, size_t i, float f)
+    {
+        reinterpret_cast<uint16_t *>(p)[i] = static_cast<uint16_t>(pack_bf16(f, 0.0f) & 0xFFFFu);
+    }
+};
+
+// fp32 sums: four accumulators per vector, no final rounding.
+struct F32Sum {
+    static constexpr int kElemBytes = 4;
+    float a[4];
+
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) a[k] = 0.0f;
+    }
+    __device__ __forceinline__ void add(u32x4 v)
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) a[k] = a[k] + bits_to_f32(v[k]);
+    }
+    __device__ __forceinline__ u32x4 result() const
+    {
+        u32x4 r;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) r[k] = f32_to_bits(a[k]);
+        return r;
+    }
+    static __device__ __forceinline__ float widen(const char *p, size_t i)
+    {
+        return reinterpret_cast<const float *>(p)[i];
+    }
+    static __device__ __forceinline__ void narrow(char *p, size_t i, float f)
+    {
+        reinterpret_cast<float *>(p)[i] = f;
+    }
+};
+
+// The order in which a workgroup visits tiles.  Workgroups are handed to the 8 XCDs
+// round-robin (workgroup b runs on XCD b % 8).  Plain order: workgroup b takes tiles
+// b, b + grid, b + 2*grid, ... so neighbouring tiles land on different XCDs.
+// XCD-contiguous order: each XCD owns one contiguous eighth of the tiles and its
+// workgroups stride through that eighth, so each XCD's L2 and TLBs see one dense address
+// range per source (the host makes the grid a multiple of 8 for this order).
+struct TileWalk {
+    size_t k, step, limit, offset, ntiles;
+    __device__ __forceinline__ TileWalk(bool xcd_contiguous, size_t ntiles_) : ntiles(ntiles_)
+    {
+        const size_t b = blockIdx.x;
+        if (xcd_contiguous) {
+            limit = (ntiles + kNumXcd - 1) / kNumXcd;
+            offset = (b % kNumXcd) * limit;
+            k = b / kNumXcd;
+            step = gridDim.x / kNumXcd;
+            if (step == 0) step = 1; // cannot happen with a host-sized grid; keeps the walk finite
+        } else {
+            limit = ntiles;
+            offset = 0;
+            k = b;
+            step = gridDim.x;
+        }
+    }
+    __device__ __forceinline__ bool valid() const { return k < limit && offset + k < ntiles; }
+    __device__ __forceinline__ size_t tile() const { return offset + k; }
+    __device__ __forceinline__ void next() { k += step; }
+};
+
+// Sum NSRC sources into NDST destinations over the vector range [0, nvec), then the
+// ragged tail elements [nvec*per_vec, numel).  Work is cut into tiles of
+// tile_iters * blockDim.x * UNROLL vectors; a workgroup walks one tile front to back and
+// then jumps gridDim.x tiles ahead.  Inside an iteration a lane issues all NSRC*UNROLL
+// loads before the first add, so up to NSRC*UNROLL*16 bytes per lane are in flight.
+// Sources are added in index order into an accumulator that starts at +0.  A destination
+// may alias a source: every vector is read and written by the same lane in the same
+// iteration, reads first.
+template <class Sum, int NSRC, int NDST, int UNROLL, bool NTL, bool NTS>
+__device__ __forceinline__ void sum_range(const char *const (&src)[NSRC], char *const (&dst)[NDST],
+                                          size_t numel, int tile_iters, bool xcd_contiguous)
+{
+    constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
+    const size_t nvec = numel / per_vec;
+    const size_t span = static_cast<size_t>(blockDim.x) * UNROLL;
+    const size_t tile = span * static_cast<size_t>(tile_iters);
+    const size_t ntiles = (nvec + tile - 1) / tile;
+
+    for (TileWalk w(xcd_contiguous, ntiles); w.valid(); w.next()) {
+        const size_t t0 = w.tile() * tile;
+        const size_t t1 = (t0 + tile < nvec) ? t0 + tile : nvec;
+        for (size_t base = t0; base < t1; base += span) {
+            u32x4 v[UNROLL][NSRC];
+            if (base + span <= t1) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+                    for (int s = 0; s < NSRC; ++s)
+                        v[u][s] = load_vec<NTL>(src[s], base + static_cast<size_t>(u) * blockDim.x + threadIdx.x);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    Sum acc;
+                    acc.zero();
+#pragma unroll
+                    for (int s = 0; s < NSRC; ++s) acc.add(v[u][s]);
+                    const u32x4 r = acc.result();
+#pragma unroll
+                    for (int d = 0; d < NDST; ++d)
+                        store_vec<NTS>(dst[d], base + static_cast<size_t>(u) * blockDim.x + threadIdx.x, r);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const size_t i = base + static_cast<size_t>(u) * blockDim.x + threadIdx.x;
+                    if (i < t1) {
+                        Sum acc;
+                        acc.zero();
+#pragma unroll
+                        for (int s = 0; s < NSRC; ++s) acc.add(load_vec<NTL>(src[s], i));
+                        const u32x4 r = acc.result();
+#pragma unroll
+                        for (int d = 0; d < NDST; ++d) store_vec<NTS>(dst[d], i, r);
+                    }
+                }
+            }
+        }
+    }
+
+    // Ragged tail: fewer than per_vec elements, handled by the first lanes of workgroup 0.
+    const size_t tail0 = nvec * per_vec;
+    if (blockIdx.x == 0 && tail0 + threadIdx.x < numel) {
+        const size_t i = tail0 + threadIdx.x;
+        float acc = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NSRC; ++s) acc = acc + Sum::widen(src[s], i);
+#pragma unroll
+        for (int d = 0; d < NDST; ++d) Sum::narrow(dst[d], i, acc);
+    }
+}
+
+// Copy one source into NDST destinations over [0, nvec) vectors; same tiling as sum_range.
+template <int NDST, int UNROLL, bool NTL, bool NTS>
+__device__ __forceinline__ void copy_range(const char *src, char *const (&dst)[NDST], size_t nvec,
+                                           int tile_iters, bool xcd_contiguous)
+{
+    const size_t span = static_cast<size_t>(blockDim.x) * UNROLL;
+    const size_t tile = span * static_cast<size_t>(tile_iters);
+    const size_t ntiles = (nvec + tile - 1) / tile;
+    for (TileWalk w(xcd_contiguous, ntiles); w.valid(); w.next()) {
+        const size_t t0 = w.tile() * tile;
+        const size_t t1 = (t0 + tile < nvec) ? t0 + tile : nvec;
+        for (size_t base = t0; base < t1; base += span) {
+            if (base + span <= t1) {
+                u32x4 v[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+                    v[u] = load_vec<NTL>(src, base + static_cast<size_t>(u) * blockDim.x + threadIdx.x);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+                    for (int d = 0; d < NDST; ++d)
+                        store_vec<NTS>(dst[d], base + static_cast<size_t>(u) * blockDim.x + threadIdx.x, v[u]);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const size_t i = base + static_cast<size_t>(u) * blockDim.x + threadIdx.x;
+                    if (i < t1) {
+                        const u32x4 v = load_vec<NTL>(src, i);
+#pragma unroll
+                        for (int d = 0; d < NDST; ++d) store_vec<NTS>(dst[d], i, v);
+                    }
+                }
+            }
+        }
+    }
+}
+
+} // namespace tccl

@@ -1,0 +1,116 @@
+"""Virtual ranks on one GPU: W separate device allocations that stand in for the
+symmetric-memory peer buffers of the reference.
+
+The reference allocates one peer-mappable buffer per process with
+``_SymmetricMemory.empty_strided_p2p`` (triton_one_shot_all_reduce_no_128.py:116-122) and
+obtains the table of all W buffer addresses with ``_SymmetricMemory.rendezvous(tensor)``
+(:82), whose handle carries ``buffer_ptrs_dev``, ``rank`` and ``world_size`` (:86-91).
+Here one process owns all W buffers; ``rendezvous`` finds the group a tensor belongs to in
+a process-local registry keyed by the address of the tensor's storage.  Signal pads do not
+exist: ordering between virtual ranks is the order of work on the HIP stream.
+"""
+from __future__ import annotations
+
+import ctypes
+import weakref
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+
+
+class SymmHandle:
+    """What ``rendezvous`` returns: the view of one virtual rank onto its group."""
+
+    def __init__(self, group: "SymmGroup", rank: int):
+        self.group = group
+        self.rank = rank
+        self.world_size = group.world_size
+        self.buffer_ptrs: Tuple[int, ...] = group.buffer_ptrs
+
+    @property
+    def buffer_ptrs_host(self) -> ctypes.Array:
+        """Host array of the W device addresses, in rank order (passed by value into the
+        kernel arguments by the library)."""
+        return self.group.ptr_array
+
+
+class SymmGroup:
+    """W same-shaped buffers, one per virtual rank, each its own allocation."""
+
+    def __init__(self, tensors: Sequence[torch.Tensor]):
+        if len(tensors) < 1:
+            raise ValueError("a group needs at least one buffer")
+        first = tensors[0]
+        for t in tensors:
+            if t.shape != first.shape or t.dtype != first.dtype or t.device != first.device:
+                raise ValueError("all buffers of a group must share shape, dtype and device")
+            if not t.is_contiguous() or t.storage_offset() != 0:
+                raise ValueError("group buffers must be whole, contiguous allocations")
+        if len({t.data_ptr() for t in tensors}) != len(tensors):
+            raise ValueError("every virtual rank needs its own allocation")
+        self.tensors: List[torch.Tensor] = list(tensors)
+        self.world_size = len(tensors)
+        self.buffer_ptrs = tuple(int(t.data_ptr()) for t in tensors)
+        self.ptr_array = _lib.ptr_array(self.buffer_ptrs)
+        self.handles = [SymmHandle(self, r) for r in range(self.world_size)]
+        # double-tree bookkeeping: outputs produced by the collective that is in progress,
+        # waiting to be picked up by the ranks that have not called yet
+        self.pending_outputs: Dict[int, torch.Tensor] = {}
+
+    def tensor(self, rank: int) -> torch.Tensor:
+        return self.tensors[rank]
+
+
+# storage base address -> (weak group, rank)
+_registry: Dict[int, Tuple["weakref.ReferenceType[SymmGroup]", int]] = {}
+
+
+def register(tensors: Sequence[torch.Tensor]) -> SymmGroup:
+    """Declare that ``tensors[r]`` is virtual rank r's buffer of one symmetric allocation."""
+    group = SymmGroup(tensors)
+    ref = weakref.ref(group)
+    for r, t in enumerate(group.tensors):
+        _registry[int(t.data_ptr())] = (ref, r)
+    # the buffers keep their group alive for as long as any of them is alive
+    for t in group.tensors:
+        t._tccl_group = group           # noqa: SLF001 -- plain attribute on the tensor object
+    return group
+
+
+def empty_world(world_size: int, size, dtype: torch.dtype, device="cuda") -> SymmGroup:
+    """Allocate one buffer per virtual rank (each a separate ``torch.empty``) and register
+    the group: the single-GPU counterpart of every rank calling ``empty_strided_p2p``."""
+    if isinstance(size, int):
+        size = (size,)
+    tensors = [torch.empty(size, dtype=dtype, device=device) for _ in range(world_size)]
+    return register(tensors)
+
+
+def rendezvous(tensor: torch.Tensor) -> SymmHandle:
+    """Handle of the group ``tensor`` belongs to, as seen by the rank that owns it.
+
+    ``tensor`` may be a rank's whole buffer or a view that starts at its first element
+    (the reference's benchmarks pass ``tensor[:size]``, triton_reduce_scatter.py:222); the
+    element count of a collective is taken from the tensor, the addresses from the group."""
+    base = int(tensor.untyped_storage().data_ptr())
+    hit = _registry.get(base)
+    group = hit[0]() if hit is not None else None
+    if group is None:
+        raise RuntimeError("tensor does not belong to a registered symmetric group "
+                           "(allocate it with tccl_amd.empty_world or register the buffers)")
+    if tensor.data_ptr() != base:
+        raise RuntimeError("a collective must be given a view that starts at the buffer's first element")
+    if not tensor.is_contiguous():
+        raise RuntimeError("a collective must be given a contiguous view")
+    return group.handles[hit[1]]
+
+
+def unregister(group: SymmGroup) -> None:
+    """Forget a group (its buffers become ordinary tensors again)."""
+    for t in group.tensors:
+        _registry.pop(int(t.data_ptr()), None)
+        if getattr(t, "_tccl_group", None) is group:
+            del t._tccl_group
+    group.pending_outputs.clear()

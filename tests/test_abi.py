@@ -1,0 +1,94 @@
+"""The C-ABI library loads on a machine without a GPU, exports every symbol the header
+declares, and rejects bad arguments before it would launch anything."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import tccl_amd
+from tccl_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "tccl_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tccl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_loader_agree():
+    syms = declared_symbols()
+    assert len(syms) >= 20
+    assert sorted(_lib.SIGNATURES) == syms
+
+
+def test_every_declared_symbol_is_exported():
+    lib = tccl_amd.load_library()
+    for name in declared_symbols():
+        assert getattr(lib, name) is not None, name
+    assert lib.tccl_abi_version() == _lib.ABI_VERSION
+
+
+def test_error_strings():
+    lib = tccl_amd.load_library()
+    assert lib.tccl_error_string(0) == b"ok"
+    assert b"16 bytes" in lib.tccl_error_string(-2)
+    assert b"power of two" in lib.tccl_error_string(-3)
+    assert lib.tccl_error_string(-1001) not in (None, b"")
+
+
+def test_argument_checks_return_codes_without_launching():
+    """All of these return before any HIP call."""
+    lib = tccl_amd.load_library()
+    good = _lib.ptr_array([0x1000, 0x2000])
+    odd = _lib.ptr_array([0x1000, 0x2008])
+    null = _lib.ptr_array([0x1000, None])
+    out = ctypes.c_void_p(0x3000)
+    assert lib.tccl_all_reduce_sum(good, 0, out, 64, 0, None) == -1          # world
+    assert lib.tccl_all_reduce_sum(good, 9, out, 64, 0, None) == -1
+    assert lib.tccl_all_reduce_sum(good, 2, out, 64, 7, None) == -1          # dtype
+    assert lib.tccl_all_reduce_sum(good, 2, None, 64, 0, None) == -1         # NULL out
+    assert lib.tccl_all_reduce_sum(null, 2, out, 64, 0, None) == -1          # NULL source
+    assert lib.tccl_all_reduce_sum(odd, 2, out, 64, 0, None) == -2           # alignment
+    assert lib.tccl_all_reduce_sum(good, 2, ctypes.c_void_p(0x3004), 64, 0, None) == -2
+    assert lib.tccl_all_reduce_sum(good, 2, out, 0, 0, None) == 0            # empty input: nothing to do
+    assert lib.tccl_reduce_scatter_sum(good, 2, 2, out, 64, 0, None) == -1   # rank out of range
+    assert lib.tccl_reduce_scatter_sum(good, 2, -1, out, 64, 0, None) == -1
+    assert lib.tccl_reduce_scatter_sum(good, 2, 1, out, 8, 0, None) == -2    # share not 16-byte aligned
+    assert lib.tccl_reduce_scatter_sum(good, 2, 1, out, 0, 0, None) == 0
+    assert lib.tccl_all_gather(good, 2, out, 24, None) == -2
+    assert lib.tccl_all_gather(good, 0, out, 32, None) == -1
+    assert lib.tccl_all_gather(good, 2, out, 0, None) == 0
+    assert lib.tccl_tree_reduce_step(None, None, None, out, 64, 0, None) == -1
+    assert lib.tccl_tree_reduce_step(ctypes.c_void_p(0x1008), None, None, out, 64, 0, None) == -2
+    assert lib.tccl_tree_copy_step(None, out, None, 64, None) == -1
+    assert lib.tccl_tree_copy_step(ctypes.c_void_p(0x1000), out, None, 24, None) == -2
+    assert lib.tccl_tree_copy_step(ctypes.c_void_p(0x1000), out, None, 0, None) == 0
+    assert lib.tccl_tree_level(None, 1, 0, 0, None) == -1
+    assert lib.tccl_tree_level(None, 0, 9, 0, None) == -1
+    assert lib.tccl_double_tree_all_reduce(good, None, 3, 64, 0, 0, None) == -3
+    assert lib.tccl_double_tree_all_reduce(good, None, 16, 64, 0, 0, None) == -1
+    assert lib.tccl_double_tree_all_reduce(good, None, 2, 60, 0, 0, None) == -2
+    assert lib.tccl_double_tree_all_reduce(good, None, 2, 0, 0, 0, None) == 0
+    assert lib.tccl_event_create(None) == -1
+    assert lib.tccl_event_elapsed_ms(None, None, None) == -1
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libtccl_amd.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.load()
+
+
+def test_product_does_not_import_the_oracle():
+    """The shipped package never reaches into oracle/."""
+    pkg = os.path.join(ROOT, "tccl_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)

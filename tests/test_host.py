@@ -1,0 +1,79 @@
+"""Host-side logic that needs no GPU: the virtual-rank registry and the wrappers'
+preconditions (the reference's assertions, raised before anything is launched)."""
+import pytest
+import torch
+
+import tccl_amd
+
+
+def make_group(world=4, numel=64, dtype=torch.bfloat16):
+    return tccl_amd.register([torch.zeros(numel, dtype=dtype) for _ in range(world)])
+
+
+def test_rendezvous_finds_rank_and_peers():
+    g = make_group(4)
+    for r in range(4):
+        h = tccl_amd.rendezvous(g.tensor(r))
+        assert h.rank == r and h.world_size == 4
+        assert h.buffer_ptrs == tuple(t.data_ptr() for t in g.tensors)
+        assert list(h.buffer_ptrs_host) == list(h.buffer_ptrs)
+    tccl_amd.unregister(g)
+
+
+def test_rendezvous_accepts_prefix_views_only():
+    g = make_group(2, 128)
+    t = g.tensor(1)
+    assert tccl_amd.rendezvous(t[:32]).rank == 1            # triton_reduce_scatter.py:222 passes tensor[:size]
+    assert tccl_amd.rendezvous(t.view(2, 64)).rank == 1
+    with pytest.raises(RuntimeError, match="first element"):
+        tccl_amd.rendezvous(t[8:])
+    with pytest.raises(RuntimeError, match="contiguous"):
+        tccl_amd.rendezvous(t[::2])
+    with pytest.raises(RuntimeError, match="registered"):
+        tccl_amd.rendezvous(torch.zeros(8))
+    tccl_amd.unregister(g)
+    with pytest.raises(RuntimeError, match="registered"):
+        tccl_amd.rendezvous(t)
+
+
+def test_group_validation():
+    a = torch.zeros(16)
+    with pytest.raises(ValueError, match="own allocation"):
+        tccl_amd.register([a, a])
+    with pytest.raises(ValueError, match="share shape"):
+        tccl_amd.register([torch.zeros(16), torch.zeros(8)])
+    with pytest.raises(ValueError, match="whole"):
+        tccl_amd.register([torch.zeros(16)[4:], torch.zeros(12)])
+    with pytest.raises(ValueError):
+        tccl_amd.register([])
+
+
+def test_wrapper_preconditions_match_the_reference():
+    """triton_one_shot_all_reduce_no_128.py:73-76, triton_reduce_scatter.py:101-104,
+    triton_all_gather.py:73-75, triton_double_tree_allreduce.py:344-347."""
+    g = make_group(4, 64, torch.bfloat16)
+    t = g.tensor(0)
+    with pytest.raises(AssertionError, match="128-bit aligned"):
+        tccl_amd.one_shot_all_reduce(t[:12])
+    with pytest.raises(AssertionError, match="128-bit aligned"):
+        tccl_amd.one_shot_reduce_scatter(t[:40])        # 40 % (8*4) != 0
+    with pytest.raises(AssertionError, match="128-bit aligned"):
+        tccl_amd.one_shot_all_gather(t[:12], 4)
+    with pytest.raises(AssertionError, match="128-bit aligned"):
+        tccl_amd.double_tree_all_reduce(t[:12])
+    with pytest.raises(AssertionError, match="world_size"):
+        tccl_amd.one_shot_all_gather(t, 8)
+    tccl_amd.unregister(g)
+    gi = make_group(2, 64, torch.int32)
+    with pytest.raises(AssertionError, match="bfloat16"):
+        tccl_amd.one_shot_all_reduce(gi.tensor(0))
+    with pytest.raises(AssertionError, match="bfloat16"):
+        tccl_amd.one_shot_reduce_scatter(gi.tensor(0))
+    with pytest.raises(AssertionError, match="bfloat16"):
+        tccl_amd.double_tree_all_reduce(gi.tensor(0))
+    tccl_amd.unregister(gi)
+
+
+def test_names():
+    assert tccl_amd.reduce_scatter is tccl_amd.one_shot_reduce_scatter
+    assert tccl_amd.all_gather is tccl_amd.one_shot_all_gather

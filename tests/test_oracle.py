@@ -1,0 +1,301 @@
+"""Pins the CPU oracle: three independent restatements (torch CPU, plain C, numpy brute
+force) against known answers the reference holds, closed forms and each other."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bit_equal, bf16_bits_equal_nan_aware, from_np_bits, np_bits, seeded_int8, seeded_randn, seeded_uniform
+from oracle import np_brute, torch_ref
+
+
+# ------------------------------------------------------------------ bf16 rounding
+
+def test_bf16_rounding_exhaustive_upper_halves(c_oracle):
+    """Every 16-bit upper half combined with lower halves on and around the rounding
+    boundary: C oracle and numpy brute force against torch's float32 -> bfloat16."""
+    upper = np.arange(1 << 16, dtype=np.uint32) << 16
+    lowers = np.array([0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF], dtype=np.uint32)
+    u = (upper[:, None] | lowers[None, :]).reshape(-1)
+    f = u.view(np.float32)
+    want = np_bits(torch.from_numpy(f.copy()).to(torch.bfloat16))
+    got_np = np_brute.narrow(f)
+    lib = c_oracle.lib()
+    isnan = np.isnan(f)
+    # NaN encodings are not part of the contract: torch's CPU conversion writes 0xFFFF for
+    # every NaN, the oracles write the canonical quiet NaN 0x7FC0.  Compare NaN-ness there.
+    assert ((want[isnan] & 0x7FFF) > 0x7F80).all()
+    assert (got_np[isnan] == 0x7FC0).all()
+    assert np.array_equal(got_np[~isnan], want[~isnan])
+    sample = np.flatnonzero(~isnan)[::97]
+    got_c = np.array([lib.orc_bf16_from_f32(float(f[i])) for i in sample], dtype=np.uint16)
+    assert np.array_equal(got_c, want[sample])
+    # a NaN cannot be handed to the C function by value without the x87/SSE path possibly
+    # quieting it, so its NaN branch is exercised through a sum instead: inf + -inf
+    inf = np.array([0x7F80], dtype=np.uint16)
+    ninf = np.array([0xFF80], dtype=np.uint16)
+    assert c_oracle.all_reduce_bf16([inf, ninf])[0] == 0x7FC0
+
+
+def test_bf16_ties_to_even():
+    # 1.0 = 0x3F80; halfway to the next bf16 is 0x3F808000 -> stays (even); 0x3F818000 -> up
+    cases = {0x3F808000: 0x3F80, 0x3F818000: 0x3F82, 0x3F808001: 0x3F81, 0x3F807FFF: 0x3F80,
+             0x7F7FFFFF: 0x7F80, 0xFF7FFFFF: 0xFF80, 0x00008000: 0x0000, 0x00018000: 0x0002,
+             0x80000000: 0x8000}
+    for src, want in cases.items():
+        f = np.array([src], dtype=np.uint32).view(np.float32)
+        assert int(np_brute.narrow(f)[0]) == want, hex(src)
+
+
+def test_widen_is_exact(c_oracle):
+    all_bits = np.arange(1 << 16, dtype=np.uint16)
+    want = from_np_bits(all_bits).float().numpy().view(np.uint32)
+    assert np.array_equal(np_brute.widen(all_bits).view(np.uint32), want)
+    lib = c_oracle.lib()
+    for b in (0x0000, 0x8000, 0x3F80, 0x0001, 0x7F80, 0xFF80, 0x7F7F):
+        got = np.array([lib.orc_f32_from_bf16(b)], dtype=np.float32).view(np.uint32)[0]
+        assert got == want[b]
+
+
+# ------------------------------------------------------------------ sums: known answers
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_fill_rank_known_answer(world, c_oracle):
+    """triton_one_shot_all_reduce_no_128.py:116-127: every rank fills 8192 elements with its
+    rank; every output element equals W(W-1)/2."""
+    bufs = [torch.full((8192,), float(r), dtype=torch.bfloat16) for r in range(world)]
+    want = world * (world - 1) // 2
+    assert torch_ref.all_reduce(bufs).eq(want).all()
+    assert from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs])).eq(want).all()
+    assert from_np_bits(np_brute.all_reduce_bf16([np_bits(b)[:64] for b in bufs])).eq(want).all()
+    # the reference's own stepwise arithmetic gives the same here (exact in bf16)
+    assert torch_ref.all_reduce_stepwise(bufs).eq(want).all()
+    for r in range(world):
+        assert torch_ref.reduce_scatter(bufs, r).eq(want).all()
+    outs = torch_ref.double_tree_all_reduce(bufs)
+    assert all(o.eq(want).all() for o in outs)
+
+
+def test_order_sensitivity_vector(c_oracle):
+    """[2^24, 1, 1, 1, 1, 1, 1, -2^24] summed in fp32 in rank order is 0 (each +1 is lost
+    against 2^24); any order that adds the ones together first is not.  Pins 'fixed rank
+    order, fp32 accumulator, no reassociation'."""
+    vals = [2.0 ** 24, 1, 1, 1, 1, 1, 1, -(2.0 ** 24)]
+    bufs = [torch.full((16,), v, dtype=torch.bfloat16) for v in vals]
+    assert torch_ref.all_reduce(bufs).eq(0).all()
+    assert from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs])).eq(0).all()
+    assert from_np_bits(np_brute.all_reduce_bf16([np_bits(b) for b in bufs])).eq(0).all()
+    rotated = [bufs[i] for i in (1, 2, 3, 4, 5, 6, 0, 7)]          # ones first: 6 + 2^24 - 2^24 = 6
+    assert torch_ref.all_reduce(rotated).eq(6).all()
+    assert from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in rotated])).eq(6).all()
+    f32 = [torch.full((16,), v, dtype=torch.float32) for v in vals]
+    assert torch_ref.all_reduce(f32).eq(0).all()
+    assert torch.from_numpy(c_oracle.all_reduce_f32([b.numpy() for b in f32])).eq(0).all()
+
+
+def test_single_rounding_not_stepwise(c_oracle):
+    """1 + 2^-8 + 2^-8: fp32 accumulation gives 1 + 2^-7 exactly (a bf16 value); re-rounding
+    after each add (the reference's add.bf16x2 arithmetic) loses both small terms."""
+    bufs = [torch.full((8,), v, dtype=torch.bfloat16) for v in (1.0, 2.0 ** -8, 2.0 ** -8)]
+    want = 1.0 + 2.0 ** -7
+    assert torch_ref.all_reduce(bufs).float().eq(want).all()
+    assert from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs])).float().eq(want).all()
+    assert from_np_bits(np_brute.all_reduce_bf16([np_bits(b) for b in bufs])).float().eq(want).all()
+    assert torch_ref.all_reduce_stepwise(bufs).float().eq(1.0).all()
+    assert from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs], stepwise=True)).float().eq(1.0).all()
+
+
+def test_zero_start_turns_negative_zero_positive(c_oracle):
+    """The accumulator starts at +0 (AR:57): a column of -0 sums to +0."""
+    bufs = [torch.full((8,), -0.0, dtype=torch.bfloat16) for _ in range(4)]
+    assert np.array_equal(np_bits(torch_ref.all_reduce(bufs)), np.zeros(8, np.uint16))
+    assert np.array_equal(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs]), np.zeros(8, np.uint16))
+    assert np.array_equal(np_brute.all_reduce_bf16([np_bits(b) for b in bufs]), np.zeros(8, np.uint16))
+    one = torch.full((8,), -0.0, dtype=torch.bfloat16)
+    assert np.array_equal(np_bits(torch_ref.tree_reduce_step(one, None, None)), np.zeros(8, np.uint16))
+
+
+def test_small_integers_exact(c_oracle):
+    """Integer inputs with |sum| <= 256 are exact in bf16 under any arithmetic."""
+    g = torch.Generator().manual_seed(7)
+    ints = [torch.randint(-16, 17, (4096,), generator=g) for _ in range(8)]
+    bufs = [i.to(torch.bfloat16) for i in ints]
+    want = sum(ints).to(torch.bfloat16)
+    assert_bit_equal(torch_ref.all_reduce(bufs), want, "torch_ref")
+    assert_bit_equal(from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs])), want, "c")
+
+
+# ------------------------------------------------------------------ sums: cross-checks
+
+DIRECTED = [0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x0080, 0x7F7F, 0xFF7F, 0x7F80, 0xFF80,
+            0x3F80, 0xBF80, 0x3F81, 0x4B80, 0xCB80, 0x3380, 0x0100, 0x8100]
+
+
+def directed_bufs(world):
+    """Columns mixing subnormals, extremes, infinities and cancellation."""
+    rng = np.random.default_rng(3)
+    cols = 512
+    out = []
+    for r in range(world):
+        pick = rng.integers(0, len(DIRECTED), size=cols)
+        out.append(np.array(DIRECTED, dtype=np.uint16)[pick])
+    return out
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 8])
+def test_three_oracles_agree_random_and_directed(world, c_oracle):
+    rand = [np_bits(t) for t in seeded_randn(world, 2048)]
+    for bufs in (rand, directed_bufs(world)):
+        t = np_bits(torch_ref.all_reduce([from_np_bits(b) for b in bufs]))
+        c = c_oracle.all_reduce_bf16(bufs)
+        n = np_brute.all_reduce_bf16(bufs)
+        assert np.array_equal(c, n)                       # both write the canonical NaN
+        assert bf16_bits_equal_nan_aware(t, c)            # torch writes 0xFFFF for NaN
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_f32_oracles_agree(world, c_oracle):
+    bufs = seeded_uniform(world, 4096)
+    t = torch_ref.all_reduce(bufs).numpy()
+    c = c_oracle.all_reduce_f32([b.numpy() for b in bufs])
+    n = np_brute.all_reduce_f32([b.numpy()[:1024] for b in bufs])
+    assert np.array_equal(t.view(np.uint32), c.view(np.uint32))
+    assert np.array_equal(t[:1024].view(np.uint32), n.view(np.uint32))
+
+
+def test_torch_ref_matches_c_at_config1_size(c_oracle):
+    """BASELINE config 1 shape: W=8 buffers of 4,194,304 bf16 ~N(0,1), seed = rank."""
+    bufs = seeded_randn(8, 4_194_304)
+    t = torch_ref.all_reduce(bufs)
+    c = c_oracle.all_reduce_bf16([np_bits(b) for b in bufs])
+    assert np.array_equal(np_bits(t), c)
+    # information only: how far the reference's stepwise arithmetic is from the contract
+    s = c_oracle.all_reduce_bf16([np_bits(b) for b in bufs], stepwise=True)
+    frac = float((s != c).mean())
+    assert 0.3 < frac < 0.7          # about half the elements differ; never a gate for the product
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_reduce_scatter_is_a_slice_of_all_reduce(world, c_oracle):
+    numel = 8 * world * 37
+    bufs = seeded_randn(world, numel)
+    full = torch_ref.all_reduce(bufs)
+    per = numel // world
+    for r in range(world):
+        assert_bit_equal(torch_ref.reduce_scatter(bufs, r), full[r * per:(r + 1) * per], f"torch r={r}")
+        got = c_oracle.reduce_scatter([np_bits(b) for b in bufs], r)
+        assert np.array_equal(got, np_bits(full[r * per:(r + 1) * per]))
+    f32 = seeded_uniform(world, numel)
+    full32 = torch_ref.all_reduce(f32)
+    for r in range(world):
+        got = c_oracle.reduce_scatter([b.numpy() for b in f32], r)
+        assert np.array_equal(got.view(np.uint32), full32[r * per:(r + 1) * per].numpy().view(np.uint32))
+
+
+def test_all_gather_of_reduce_scatter_is_all_reduce():
+    """Slide 'Triton all-gather': reduce-scatter then all-gather composes to all-reduce."""
+    world, numel = 8, 8 * 8 * 16
+    bufs = seeded_randn(world, numel)
+    shares = [torch_ref.reduce_scatter(bufs, r) for r in range(world)]
+    assert_bit_equal(torch_ref.all_gather(shares).reshape(-1), torch_ref.all_reduce(bufs), "AG o RS")
+
+
+# ------------------------------------------------------------------ gather / copy
+
+@pytest.mark.parametrize("maker,name", [(seeded_randn, "bf16"), (seeded_uniform, "f32"), (seeded_int8, "int8")])
+def test_all_gather_equals_stack(maker, name, c_oracle):
+    """triton_all_gather.py:128: expected value is the stack of the sources."""
+    world, numel = 8, 4096
+    bufs = maker(world, numel)
+    want = torch.stack(bufs)
+    assert_bit_equal(torch_ref.all_gather(bufs), want, name)
+    raw = [b.view(torch.uint8).numpy() for b in bufs]
+    got = c_oracle.all_gather(raw)
+    assert np.array_equal(got.reshape(-1), want.view(torch.uint8).numpy().reshape(-1))
+
+
+def test_tree_copy_step_oracle(c_oracle):
+    src = np.arange(4096, dtype=np.uint16)
+    d0, d1 = c_oracle.tree_copy_step(src, 2)
+    assert np.array_equal(d0, src) and np.array_equal(d1, src)
+
+
+# ------------------------------------------------------------------ tree step and full tree
+
+@pytest.mark.parametrize("children", [(False, False), (True, False), (False, True), (True, True)])
+def test_tree_reduce_step_oracles_agree(children, c_oracle):
+    own, c0, c1 = [np_bits(t) for t in seeded_randn(3, 2048, seed_base=11)]
+    k0 = c0 if children[0] else None
+    k1 = c1 if children[1] else None
+    t = np_bits(torch_ref.tree_reduce_step(from_np_bits(own), from_np_bits(k0) if k0 is not None else None,
+                                           from_np_bits(k1) if k1 is not None else None))
+    assert np.array_equal(t, c_oracle.tree_reduce_step(own, k0, k1))
+    assert np.array_equal(t, np_brute.tree_reduce_step_bf16(own, k0, k1))
+    # the step is the ordered sum (child0, child1, own)
+    srcs = [x for x in (k0, k1) if x is not None] + [own]
+    assert np.array_equal(t, c_oracle.all_reduce_bf16(srcs))
+
+
+@pytest.mark.parametrize("world", [2, 4, 8, 16])
+@pytest.mark.parametrize("numel", [16, 8 * 123, 65536 + 8])
+def test_double_tree_c_vs_recursive_torch(world, numel, c_oracle):
+    """Level-ordered in-place sweep (C) against the recursion over the rank graph (torch):
+    different traversals, same rule."""
+    bufs = seeded_randn(world, numel, seed_base=100)
+    want = torch_ref.double_tree_all_reduce(bufs)
+    final, outs = c_oracle.double_tree_all_reduce_bf16([np_bits(b) for b in bufs])
+    for r in range(world):
+        assert np.array_equal(outs[r], np_bits(want[r])), r
+        assert np.array_equal(final[r], outs[r]), r           # buffers end up holding the result
+    for r in range(1, world):
+        assert np.array_equal(outs[r], outs[0])               # all ranks bit-identical
+
+
+def test_double_tree_order_is_the_tree_order():
+    """W=8, tree a: ((x1 + x3 + x2) + (x5 + x7 + x6) + x4) + x0 with a rounding after every
+    bracket; written out by hand for one half, from the tree picture in tree.py:56-63."""
+    bufs = seeded_randn(8, 64, seed_base=5)
+    split = torch_ref.double_tree_split(64, 2)
+    assert split == 32
+    x = [b[:split] for b in bufs]
+
+    def rnd(*terms):
+        acc = torch.zeros(split, dtype=torch.float32)
+        for t in terms:
+            acc += t
+        return acc.to(torch.bfloat16)
+    r2 = rnd(rnd(x[1]), rnd(x[3]), x[2])
+    r6 = rnd(rnd(x[5]), rnd(x[7]), x[6])
+    r4 = rnd(r2, r6, x[4])
+    r0 = rnd(r4, x[0])
+    got = torch_ref.double_tree_all_reduce(bufs)[3]
+    assert_bit_equal(got[:split], r0, "tree a by hand")
+    y = [b[split:] for b in bufs]
+    split2 = 64 - split
+
+    def rnd2(*terms):
+        acc = torch.zeros(split2, dtype=torch.float32)
+        for t in terms:
+            acc += t
+        return acc.to(torch.bfloat16)
+    r1 = rnd2(rnd2(y[0]), rnd2(y[2]), y[1])
+    r5 = rnd2(rnd2(y[4]), rnd2(y[6]), y[5])
+    r3 = rnd2(r1, r5, y[3])
+    r7 = rnd2(r3, y[7])
+    assert_bit_equal(got[split:], r7, "tree b by hand")
+
+
+def test_double_tree_differs_from_flat_sum_only_slightly():
+    """One rounding per level: close to the flat fp32 sum, not identical to it."""
+    bufs = seeded_randn(8, 1 << 16, seed_base=0)
+    flat = torch_ref.all_reduce(bufs).float()
+    tree = torch_ref.double_tree_all_reduce(bufs)[0].float()
+    diff = (flat - tree).abs()
+    assert (diff > 0).any()
+    assert (diff <= 0.0625 * flat.abs().clamp(min=1.0)).all()
+
+
+def test_double_tree_split():
+    assert torch_ref.double_tree_split(134_217_728, 2) == 67_108_864
+    assert torch_ref.double_tree_split(24, 2) == 8
+    assert torch_ref.double_tree_split(8, 2) == 0
+    assert torch_ref.double_tree_split(10, 4) == 4

@@ -1,0 +1,415 @@
+"""GPU parity: every HIP kernel, called through the C ABI (directly or via the host
+wrappers, which only add allocation and argument checks), against the CPU oracle on the
+same seeded inputs.  Bit-exact unless stated."""
+import ctypes
+import gc
+
+import numpy as np
+import pytest
+import torch
+
+import tccl_amd
+from tccl_amd import _lib
+from helpers import (assert_bit_equal, assert_bit_equal_nan_aware, from_np_bits, np_bits, seeded_int8,
+                     seeded_randn, seeded_uniform)
+from oracle import torch_ref
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(autouse=True)
+def _gpu_hygiene():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    tccl_amd.load_library()
+    groups = []
+    yield groups
+    torch.cuda.synchronize()
+    for g in groups:
+        tccl_amd.unregister(g)
+    groups.clear()
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def upload(groups, bufs):
+    """One separate device allocation per virtual rank, filled from the CPU tensors."""
+    g = tccl_amd.empty_world(len(bufs), bufs[0].shape, bufs[0].dtype, DEV)
+    for r, b in enumerate(bufs):
+        g.tensor(r).copy_(b)
+    groups.append(g)
+    return g
+
+
+def stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def oracle_sum(c_oracle, bufs):
+    if bufs[0].dtype == torch.bfloat16:
+        return from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs]))
+    return torch.from_numpy(c_oracle.all_reduce_f32([b.numpy() for b in bufs]))
+
+
+# ------------------------------------------------------------------ one-shot all-reduce
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_all_reduce_fill_rank(world, _gpu_hygiene):
+    """The reference's own test, triton_one_shot_all_reduce_no_128.py:116-127."""
+    g = upload(_gpu_hygiene, [torch.full((8192,), float(r), dtype=torch.bfloat16) for r in range(world)])
+    for r in range(world):
+        out = tccl_amd.one_shot_all_reduce(g.tensor(r))
+        assert out.eq(world * (world - 1) // 2).all().item()
+        assert out.dtype == torch.bfloat16 and out.shape == (8192,)
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+def test_all_reduce_matches_oracle(world, maker, _gpu_hygiene, c_oracle):
+    numel = 8 * 40_003                       # many tiles plus a partial one
+    bufs = maker(world, numel)
+    g = upload(_gpu_hygiene, bufs)
+    want = oracle_sum(c_oracle, bufs)
+    assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0)), want, f"W={world}")
+
+
+@pytest.mark.parametrize("numel", [0, 1, 7, 8, 9, 515, 2048 * 8 + 5, 1_000_003])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+def test_all_reduce_ragged_sizes_through_c_abi(numel, maker, _gpu_hygiene, c_oracle):
+    """Sizes that are not whole 16-byte vectors: the wrappers refuse them as the reference
+    does, the C entry point sums the tail one element at a time."""
+    world = 4
+    bufs = maker(world, max(numel, 8))
+    g = upload(_gpu_hygiene, bufs)
+    out = torch.full((max(numel, 8) + 8,), 77.0, dtype=bufs[0].dtype, device=DEV)
+    dt = _lib.TCCL_BF16 if bufs[0].dtype == torch.bfloat16 else _lib.TCCL_F32
+    rc = tccl_amd.load_library().tccl_all_reduce_sum(g.ptr_array, world, out.data_ptr(), numel, dt, stream())
+    assert rc == 0
+    want = oracle_sum(c_oracle, [b[:numel].contiguous() for b in bufs]) if numel else bufs[0][:0]
+    assert_bit_equal(out[:numel], want, f"numel={numel}")
+    assert out[numel:].eq(77.0).all().item(), "wrote past the end"
+
+
+@pytest.mark.parametrize("block", [64, 128, 256, 512])
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+@pytest.mark.parametrize("flags", [0, 1, 2, 3, 4, 7])
+def test_all_reduce_every_launch_shape(block, unroll, flags, _gpu_hygiene, c_oracle):
+    """Every kernel instantiation and tiling mode gives the same bits."""
+    bufs = seeded_randn(8, 8 * 30_011)
+    g = upload(_gpu_hygiene, bufs)
+    want = oracle_sum(c_oracle, bufs)
+    for tile_iters, grid in ((0, 0), (4, 0), (1, 24), (3, 40), (16, 8)):
+        cfg = tccl_amd.LaunchCfg(block=block, unroll=unroll, grid=grid, tile_iters=tile_iters, flags=flags)
+        got = tccl_amd.one_shot_all_reduce(g.tensor(0), cfg=cfg)
+        assert_bit_equal(got, want, f"block={block} unroll={unroll} flags={flags} tile={tile_iters} grid={grid}")
+    small = seeded_randn(3, 8 * 1001)
+    g3 = upload(_gpu_hygiene, small)
+    cfg = tccl_amd.LaunchCfg(block=block, unroll=unroll, flags=flags)
+    assert_bit_equal(tccl_amd.one_shot_all_reduce(g3.tensor(0), cfg=cfg), oracle_sum(c_oracle, small), "W=3")
+
+
+def test_all_reduce_order_and_single_rounding(_gpu_hygiene):
+    """fp32 accumulation in rank order: [2^24, 1 x6, -2^24] -> 0; ones first -> 6;
+    1 + 2^-8 + 2^-8 -> 1 + 2^-7 (a bf16-stepwise sum would give 1)."""
+    vals = [2.0 ** 24, 1, 1, 1, 1, 1, 1, -(2.0 ** 24)]
+    for dtype in (torch.bfloat16, torch.float32):
+        g = upload(_gpu_hygiene, [torch.full((4096,), v, dtype=dtype) for v in vals])
+        assert tccl_amd.one_shot_all_reduce(g.tensor(0)).eq(0).all().item()
+        rot = upload(_gpu_hygiene, [torch.full((4096,), vals[i], dtype=dtype) for i in (1, 2, 3, 4, 5, 6, 0, 7)])
+        assert tccl_amd.one_shot_all_reduce(rot.tensor(0)).eq(6).all().item()
+    g = upload(_gpu_hygiene, [torch.full((4096,), v, dtype=torch.bfloat16) for v in (1.0, 2.0 ** -8, 2.0 ** -8)])
+    assert tccl_amd.one_shot_all_reduce(g.tensor(0)).float().eq(1.0 + 2.0 ** -7).all().item()
+
+
+def test_all_reduce_directed_bit_patterns(_gpu_hygiene, c_oracle):
+    """Subnormals (kept, not flushed), signed zeros (+0 start), infinities, overflow to
+    infinity, round-to-nearest-even ties, NaN (any NaN encoding accepted)."""
+    pats = np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x0080, 0x7F7F, 0xFF7F, 0x7F80, 0xFF80, 0x3F80,
+                     0xBF80, 0x3F81, 0x4B80, 0xCB80, 0x3380, 0x0100, 0x8100, 0x7FC0, 0xFFC1], dtype=np.uint16)
+    rng = np.random.default_rng(5)
+    for world in (2, 3, 8):
+        bufs = [from_np_bits(pats[rng.integers(0, len(pats), size=8 * 4096)]) for _ in range(world)]
+        g = upload(_gpu_hygiene, bufs)
+        want = oracle_sum(c_oracle, bufs)
+        assert_bit_equal_nan_aware(tccl_amd.one_shot_all_reduce(g.tensor(0)), want, f"W={world}")
+    # ties: 1 + 2^-8 is halfway between bf16 1.0 and 1+2^-7 -> even (1.0); 1+2^-7 + 2^-8 -> 1+2^-6
+    for base, want in ((1.0, 1.0), (1.0 + 2.0 ** -7, 1.0 + 2.0 ** -6)):
+        g = upload(_gpu_hygiene, [torch.full((64,), base, dtype=torch.bfloat16),
+                                  torch.full((64,), 2.0 ** -8, dtype=torch.bfloat16)])
+        assert tccl_amd.one_shot_all_reduce(g.tensor(0)).float().eq(want).all().item()
+    # -0 + -0 -> +0 because the accumulator starts at +0
+    g = upload(_gpu_hygiene, [torch.full((64,), -0.0, dtype=torch.bfloat16) for _ in range(2)])
+    assert np.array_equal(np_bits(tccl_amd.one_shot_all_reduce(g.tensor(0))), np.zeros(64, np.uint16))
+    # fp32 subnormals survive
+    tiny = torch.full((64,), 1e-45, dtype=torch.float32)
+    g = upload(_gpu_hygiene, [tiny.clone(), tiny.clone()])
+    assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0)), tiny + tiny, "fp32 subnormal")
+
+
+def test_all_reduce_config1_vs_torch_cpu_reference(_gpu_hygiene, c_oracle):
+    """BASELINE config 1: W=8 x 4,194,304 bf16 ~N(0,1), seed = rank, against the torch CPU
+    reference (and the C oracle)."""
+    bufs = seeded_randn(8, 4_194_304)
+    g = upload(_gpu_hygiene, bufs)
+    want = torch_ref.all_reduce(bufs)
+    for r in (0, 5):
+        assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(r)), want, f"rank {r}")
+    assert_bit_equal(oracle_sum(c_oracle, bufs), want, "oracles")
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_all_reduce_sweep_sizes(world, _gpu_hygiene, c_oracle):
+    """BASELINE config 2 sweep: 16 KiB .. 64 MiB per buffer in powers of 4, using prefix
+    views of one allocation (as the reference's benchmarks slice tensor[:size])."""
+    top = (64 << 20) // 2
+    bufs = seeded_randn(world, top)
+    g = upload(_gpu_hygiene, bufs)
+    nbytes = 16 << 10
+    while nbytes <= (64 << 20):
+        n = nbytes // 2
+        want = oracle_sum(c_oracle, [b[:n] for b in bufs])
+        assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(1)[:n]), want, f"W={world} {nbytes} B")
+        nbytes *= 4
+
+
+def test_all_reduce_256mib_per_buffer(_gpu_hygiene, c_oracle):
+    """Largest sweep point: 8 x 256 MiB (offsets beyond 2^31 bytes in total)."""
+    n = (256 << 20) // 2
+    torch.manual_seed(0)
+    base = torch.randn(n, dtype=torch.bfloat16)
+    bufs = [base.roll(r * 1_000_003) for r in range(8)]
+    g = upload(_gpu_hygiene, bufs)
+    out = tccl_amd.one_shot_all_reduce(g.tensor(0))
+    want = oracle_sum(c_oracle, bufs)
+    assert_bit_equal(out, want, "256 MiB")
+
+
+# ------------------------------------------------------------------ reduce-scatter
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+def test_reduce_scatter_every_rank(world, maker, _gpu_hygiene, c_oracle):
+    numel = 8 * world * 5_003
+    bufs = maker(world, numel)
+    g = upload(_gpu_hygiene, bufs)
+    full = oracle_sum(c_oracle, bufs)
+    per = numel // world
+    ar = tccl_amd.one_shot_all_reduce(g.tensor(0))
+    shares = []
+    for r in range(world):
+        got = tccl_amd.reduce_scatter(g.tensor(r))
+        assert got.shape == (per,)
+        assert_bit_equal(got, full[r * per:(r + 1) * per], f"rank {r}")
+        assert_bit_equal(got, ar[r * per:(r + 1) * per], f"rank {r} vs all-reduce slice")
+        shares.append(got)
+    # all-gather of the shares is the all-reduce
+    gs = tccl_amd.register(shares)
+    _gpu_hygiene.append(gs)
+    assert_bit_equal(tccl_amd.all_gather(shares[0], world).reshape(-1), ar, "AG o RS")
+
+
+def test_reduce_scatter_config3(_gpu_hygiene, c_oracle):
+    """BASELINE config 3: W=8 inputs of 67,108,864 bf16 ~N(0,1), rank 3's 8,388,608-element
+    share; then the same shapes in fp32 ~U(-1,1)."""
+    world, numel, rank = 8, 67_108_864, 3
+    per = numel // world
+    for maker in (seeded_randn, seeded_uniform):
+        bufs = maker(world, numel)
+        g = upload(_gpu_hygiene, bufs)
+        got = tccl_amd.reduce_scatter(g.tensor(rank))
+        want = oracle_sum(c_oracle, [b[rank * per:(rank + 1) * per].contiguous() for b in bufs])
+        assert_bit_equal(got, want, maker.__name__)
+        tccl_amd.unregister(g)
+        _gpu_hygiene.remove(g)
+        del g, got, bufs
+        gc.collect()
+        torch.cuda.empty_cache()
+
+
+def test_reduce_scatter_fill_rank(_gpu_hygiene):
+    g = upload(_gpu_hygiene, [torch.full((8 * 8 * 64,), float(r), dtype=torch.bfloat16) for r in range(8)])
+    for r in range(8):
+        assert tccl_amd.reduce_scatter(g.tensor(r)).eq(28).all().item()
+
+
+# ------------------------------------------------------------------ all-gather
+
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform, seeded_int8], ids=["bf16", "f32", "int8"])
+@pytest.mark.parametrize("numel", [16, 4096, 8_388_608])
+def test_all_gather_equals_stack(maker, numel, _gpu_hygiene):
+    """BASELINE config 4 (numel = 8,388,608) and smaller; expected value as in
+    triton_all_gather.py:128."""
+    world = 8
+    bufs = maker(world, numel)
+    g = upload(_gpu_hygiene, bufs)
+    out = tccl_amd.all_gather(g.tensor(2), world)
+    assert out.shape == (world, numel) and out.dtype == bufs[0].dtype
+    assert_bit_equal(out, torch.stack(bufs), maker.__name__)
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 5, 8])
+def test_all_gather_worlds_shapes_and_nan_payloads(world, _gpu_hygiene):
+    rng = np.random.default_rng(world)
+    bufs = [from_np_bits(rng.integers(0, 1 << 16, size=(24 * 8 * 11,), dtype=np.uint16)).reshape(24, 88)
+            for _ in range(world)]                  # every bit pattern incl. NaN payloads
+    g = upload(_gpu_hygiene, bufs)
+    out = tccl_amd.one_shot_all_gather(g.tensor(0), world)
+    assert out.shape == (world, 24, 88)
+    assert_bit_equal(out, torch.stack(bufs), f"W={world}")
+
+
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+@pytest.mark.parametrize("flags", [0, 3, 4])
+def test_all_gather_launch_shapes(unroll, flags, _gpu_hygiene):
+    bufs = seeded_int8(4, 16 * 70_001)
+    g = upload(_gpu_hygiene, bufs)
+    for block, tile_iters, grid in ((64, 0, 0), (256, 5, 16), (512, 1, 3)):
+        cfg = tccl_amd.LaunchCfg(block=block, unroll=unroll, grid=grid, tile_iters=tile_iters, flags=flags)
+        assert_bit_equal(tccl_amd.all_gather(g.tensor(0), 4, cfg=cfg), torch.stack(bufs), f"{block}/{unroll}")
+
+
+# ------------------------------------------------------------------ double-tree node steps
+
+@pytest.mark.parametrize("children", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+@pytest.mark.parametrize("in_place", [False, True])
+def test_tree_reduce_step(children, maker, in_place, _gpu_hygiene, c_oracle):
+    numel = 65_536 * 3 + 8 * 5                      # three 128 KiB chunks (bf16) and a bit
+    own, c0, c1 = maker(3, numel, seed_base=40)
+    k0 = c0 if children[0] else None
+    k1 = c1 if children[1] else None
+    want = torch_ref.tree_reduce_step(own, k0, k1)
+    d_own, d0, d1 = own.to(DEV), c0.to(DEV), c1.to(DEV)
+    dst = d_own if in_place else torch.empty_like(d_own)
+    dt = _lib.TCCL_BF16 if own.dtype == torch.bfloat16 else _lib.TCCL_F32
+    rc = tccl_amd.load_library().tccl_tree_reduce_step(
+        d_own.data_ptr(), d0.data_ptr() if children[0] else None, d1.data_ptr() if children[1] else None,
+        dst.data_ptr(), numel, dt, stream())
+    assert rc == 0
+    assert_bit_equal(dst, want, f"children={children}")
+    assert_bit_equal(d0, c0, "child0 untouched")
+    assert_bit_equal(d1, c1, "child1 untouched")
+
+
+@pytest.mark.parametrize("two", [False, True])
+def test_tree_copy_step(two, _gpu_hygiene):
+    src = seeded_int8(1, 16 * 100_003)[0]
+    d_src = src.to(DEV)
+    a = torch.zeros_like(d_src)
+    b = torch.zeros_like(d_src)
+    rc = tccl_amd.load_library().tccl_tree_copy_step(d_src.data_ptr(), a.data_ptr(), b.data_ptr() if two else None,
+                                                     src.numel(), stream())
+    assert rc == 0
+    assert_bit_equal(a, src, "dst0")
+    assert_bit_equal(b, src if two else torch.zeros_like(src), "dst1")
+
+
+def test_tree_level_batch(_gpu_hygiene, c_oracle):
+    """Several node steps of different kinds and lengths in one launch."""
+    lib = tccl_amd.load_library()
+    n1, n2 = 65_536 * 2 + 24, 8 * 777
+    x = [t.to(DEV) for t in seeded_randn(6, n1, seed_base=60)]
+    cpu = [t.cpu().clone() for t in x]
+    outs = [torch.zeros(n1, dtype=torch.bfloat16, device=DEV) for _ in range(4)]
+    jobs = (_lib.NodeJob * 4)()
+
+    def fill(j, src, dst, numel, is_copy):
+        for k in range(3):
+            j.src[k] = src[k]
+        for k in range(2):
+            j.dst[k] = dst[k]
+        j.numel, j.is_copy = numel, is_copy
+    fill(jobs[0], [x[0].data_ptr(), x[1].data_ptr(), x[2].data_ptr()], [outs[0].data_ptr(), None], n1, 0)
+    fill(jobs[1], [x[3].data_ptr(), None, x[4].data_ptr()], [x[4].data_ptr(), outs[1].data_ptr()], n2, 0)   # in place + 2nd dst
+    fill(jobs[2], [x[5].data_ptr(), None, None], [outs[2].data_ptr(), outs[3].data_ptr()], n1, 1)
+    fill(jobs[3], [None, None, x[5].data_ptr()], [x[5].data_ptr(), None], n2, 0)           # leaf step in place, after job 2 reads? no: same launch
+    # job 3 would race with job 2 on x[5]; give it its own buffer instead
+    y = seeded_randn(1, n2, seed_base=99)[0]
+    d_y = y.to(DEV)
+    fill(jobs[3], [None, None, d_y.data_ptr()], [d_y.data_ptr(), None], n2, 0)
+    for chunk in (0, 4096, 1 << 20):
+        for o in outs:
+            o.zero_()
+        x[4].copy_(cpu[4])
+        d_y.copy_(y)
+        assert lib.tccl_tree_level(jobs, 4, _lib.TCCL_BF16, chunk, stream()) == 0
+        assert_bit_equal(outs[0], torch_ref.tree_reduce_step(cpu[2], cpu[0], cpu[1]), "job 0")
+        w1 = torch_ref.tree_reduce_step(cpu[4][:n2], cpu[3][:n2], None)
+        assert_bit_equal(x[4][:n2], w1, "job 1 in place")
+        assert_bit_equal(x[4][n2:], cpu[4][n2:], "job 1 beyond its range")
+        assert_bit_equal(outs[1][:n2], w1, "job 1 second destination")
+        assert_bit_equal(outs[2], cpu[5], "job 2 copy")
+        assert_bit_equal(outs[3], cpu[5], "job 2 copy, second destination")
+        assert_bit_equal(d_y, torch_ref.tree_reduce_step(y, None, None), "job 3")
+
+
+# ------------------------------------------------------------------ full double tree
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+@pytest.mark.parametrize("numel", [8, 16, 8 * 12_345, 65_536 * 4 + 8])
+def test_double_tree_all_ranks(world, numel, _gpu_hygiene, c_oracle):
+    bufs = seeded_randn(world, numel, seed_base=100)
+    final, outs = c_oracle.double_tree_all_reduce_bf16([np_bits(b) for b in bufs])
+    want = from_np_bits(outs[0])
+    assert_bit_equal(want, torch_ref.double_tree_all_reduce(bufs)[0], "oracles agree")
+    g = upload(_gpu_hygiene, bufs)
+    got = [tccl_amd.double_tree_all_reduce(g.tensor(r)) for r in range(world)]   # one call per rank
+    for r in range(world):
+        assert_bit_equal(got[r], want, f"output of rank {r}")
+        assert_bit_equal(g.tensor(r), from_np_bits(final[r]), f"buffer of rank {r}")
+
+
+def test_double_tree_fill_rank_and_second_collective(_gpu_hygiene):
+    world = 8
+    g = upload(_gpu_hygiene, [torch.full((8192,), float(r), dtype=torch.bfloat16) for r in range(world)])
+    for r in range(world):
+        assert tccl_amd.double_tree_all_reduce(g.tensor(r)).eq(28).all().item()
+    # every buffer now holds 28; the next collective sums those: 8 * 28
+    for r in range(world):
+        assert tccl_amd.double_tree_all_reduce(g.tensor(r)).eq(224).all().item()
+
+
+def test_double_tree_f32_and_chunk_sizes(_gpu_hygiene, c_oracle):
+    world, numel = 4, 4 * 50_001
+    bufs = seeded_uniform(world, numel, seed_base=7)
+    want = torch_ref.double_tree_all_reduce(bufs)[0]
+    for chunk in (0, 1024, 1 << 22):
+        g = upload(_gpu_hygiene, bufs)
+        outs = tccl_amd.double_tree_all_reduce_world(g, chunk_elems=chunk)
+        for r in range(world):
+            assert_bit_equal(outs[r], want, f"chunk={chunk} rank {r}")
+
+
+def test_double_tree_config5_properties(_gpu_hygiene, c_oracle):
+    """BASELINE config 5 shape: W=8 x 134,217,728 bf16 (256 MiB each), halves of
+    67,108,864 elements, 65,536-element chunks.  Checked by size-independent properties:
+    all 8 outputs and all 8 buffers are bit-identical, and windows of the result equal the
+    oracle run on the same windows of the inputs."""
+    world, numel = 8, 134_217_728
+    torch.manual_seed(0)
+    base = torch.randn(numel, dtype=torch.bfloat16)
+    g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    shifts = [r * 7_000_001 for r in range(world)]
+    dbase = base.to(DEV)
+    for r in range(world):
+        g.tensor(r).copy_(dbase.roll(shifts[r]))
+    del dbase
+    half = numel // 2
+    windows = [(0, 65_536 * 2), (half - 65_536, 65_536), (half - 8, 8), (31_457_280, 8 * 1001)]
+    samples = []
+    for lo, n in windows:
+        a = [g.tensor(r)[lo:lo + n].cpu() for r in range(world)]
+        b = [g.tensor(r)[half + lo:half + lo + n].cpu() for r in range(world)]
+        samples.append([torch.cat([x, y]) for x, y in zip(a, b)])
+    outs = tccl_amd.double_tree_all_reduce_world(g)
+    for r in range(1, world):
+        assert torch.equal(outs[r].view(torch.int16), outs[0].view(torch.int16)), f"output {r}"
+    for r in range(world):
+        assert torch.equal(g.tensor(r).view(torch.int16), outs[0].view(torch.int16)), f"buffer {r}"
+    for (lo, n), sample in zip(windows, samples):
+        _, want = c_oracle.double_tree_all_reduce_bf16([np_bits(s) for s in sample])
+        w = from_np_bits(want[0])
+        assert_bit_equal(outs[0][lo:lo + n], w[:n], f"tree a window at {lo}")
+        assert_bit_equal(outs[0][half + lo:half + lo + n], w[n:], f"tree b window at {lo}")
