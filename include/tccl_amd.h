@@ -66,6 +66,10 @@ typedef struct {
 #define TCCL_CFG_NONTEMPORAL_STORE 2 /* mark stores as streaming */
 #define TCCL_CFG_XCD_CONTIGUOUS 4    /* give each of the 8 XCDs one contiguous eighth of the tiles */
 #define TCCL_CFG_TEMPORAL 8          /* force plain (cached) loads and stores */
+#define TCCL_CFG_STREAMING 16        /* force the grid-stride kernel (stores interleaved with loads) */
+#define TCCL_CFG_PHASED 32           /* force the phased kernel (each workgroup reads its whole tile,
+                                        then writes it); there `grid` = workgroups per launch and
+                                        `tile_iters` = iterations per tile (1..16), block/unroll unused */
 
 int tccl_abi_version(void);
 const char *tccl_error_string(int code);

@@ -23,6 +23,8 @@ CFG_NONTEMPORAL_LOAD = 1
 CFG_NONTEMPORAL_STORE = 2
 CFG_XCD_CONTIGUOUS = 4
 CFG_TEMPORAL = 8
+CFG_STREAMING = 16
+CFG_PHASED = 32
 
 
 class TcclError(RuntimeError):

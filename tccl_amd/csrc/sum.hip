@@ -75,6 +75,96 @@ static hipError_t launch_sum_nsrc(const char *const *srcs, int nsrc, char *out, 
     }
 }
 
+// ---------------------------------------------------------------------------------
+// Phased variant: one tile per workgroup, all of a launch's workgroups resident at once.
+
+template <class Sum, int NSRC>
+__global__ void __launch_bounds__(kPhasedBlock)
+sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_t tail_first, size_t numel)
+{
+    constexpr int U = PhasedUnroll<NSRC>::value;
+    constexpr int KMAX = PhasedUnroll<NSRC>::kmax;
+    const size_t tile_bytes = static_cast<size_t>(kcount) * (kPhasedBlock * U * kVecBytes);
+    const size_t off = blockIdx.x * tile_bytes;
+    const size_t left = bytes > off ? bytes - off : 0;
+    const uint32_t valid = static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes);
+    char *const dst[1] = {out};
+    sum_tile_phased<Sum, NSRC, 1, U, KMAX>(src.p, dst, off, valid, kcount);
+    if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
+}
+
+template <class Sum, int NSRC>
+static hipError_t launch_phased(const char *const *srcs, char *out, size_t numel, const tccl_launch_cfg *cfg,
+                                hipStream_t stream)
+{
+    constexpr int U = PhasedUnroll<NSRC>::value;
+    constexpr size_t kPhasedKMax = PhasedUnroll<NSRC>::kmax;
+    constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
+    constexpr size_t span = static_cast<size_t>(kPhasedBlock) * U; // vectors per iteration
+    const size_t nvec = numel / per_vec;
+    size_t wgs = (cfg && cfg->grid > 0) ? static_cast<size_t>(cfg->grid) : static_cast<size_t>(compute_units()) * 2;
+    size_t kcount;
+    if (cfg && cfg->tile_iters > 0) {
+        kcount = static_cast<size_t>(cfg->tile_iters) > kPhasedKMax ? kPhasedKMax : cfg->tile_iters;
+    } else {
+        // Fewest launches that fit, then the smallest tile that covers a launch's share
+        // with `wgs` workgroups, so that every launch is one full, even wave of workgroups.
+        const size_t launches = (nvec + wgs * span * kPhasedKMax - 1) / (wgs * span * kPhasedKMax);
+        const size_t per_launch = (nvec + (launches ? launches : 1) - 1) / (launches ? launches : 1);
+        kcount = (per_launch + wgs * span - 1) / (wgs * span);
+        if (kcount < 1) kcount = 1;
+        if (kcount > kPhasedKMax) kcount = kPhasedKMax;
+    }
+    const size_t tile_vec = kcount * span;
+    const size_t slice_vec = wgs * tile_vec;
+    const size_t tail_first = nvec * per_vec;
+
+    size_t off = 0;
+    do {
+        const size_t n = nvec - off < slice_vec ? nvec - off : slice_vec;
+        const bool last = off + n >= nvec;
+        SrcTable<NSRC> t;
+        for (int i = 0; i < NSRC; ++i) t.p[i] = srcs[i] + off * kVecBytes;
+        size_t grid = (n + tile_vec - 1) / tile_vec;
+        if (grid == 0) grid = 1; // nothing but a ragged tail
+        // the tail's element indices are relative to this launch's base pointers
+        const size_t rel_first = last ? tail_first - off * per_vec : 0;
+        const size_t rel_numel = last ? numel - off * per_vec : 0;
+        hipLaunchKernelGGL((sum_phased_kernel<Sum, NSRC>), dim3(static_cast<unsigned>(grid)), dim3(kPhasedBlock), 0,
+                           stream, t, out + off * kVecBytes, n * kVecBytes, static_cast<int>(kcount), rel_first,
+                           rel_numel);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        off += n;
+    } while (off < nvec);
+    return hipSuccess;
+}
+
+template <class Sum>
+static hipError_t launch_phased_nsrc(const char *const *srcs, int nsrc, char *out, size_t numel,
+                                     const tccl_launch_cfg *cfg, hipStream_t stream)
+{
+    switch (nsrc) {
+    case 1: return launch_phased<Sum, 1>(srcs, out, numel, cfg, stream);
+    case 2: return launch_phased<Sum, 2>(srcs, out, numel, cfg, stream);
+    case 3: return launch_phased<Sum, 3>(srcs, out, numel, cfg, stream);
+    case 4: return launch_phased<Sum, 4>(srcs, out, numel, cfg, stream);
+    case 5: return launch_phased<Sum, 5>(srcs, out, numel, cfg, stream);
+    case 6: return launch_phased<Sum, 6>(srcs, out, numel, cfg, stream);
+    case 7: return launch_phased<Sum, 7>(srcs, out, numel, cfg, stream);
+    case 8: return launch_phased<Sum, 8>(srcs, out, numel, cfg, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// Inputs of at least this many output bytes take the phased kernel: below it a launch
+// cannot give every compute unit two tiles of at least two iterations.
+static size_t phased_min_bytes(int nsrc)
+{
+    const int u = nsrc <= 2 ? 8 : (nsrc <= 4 ? 4 : 2);
+    return static_cast<size_t>(compute_units()) * 2 * kPhasedBlock * u * kVecBytes * 2;
+}
+
 // Sum `nsrc` already-offset source pointers into `out`.  Shared by the three entry points.
 int sum_streams(const void *const *srcs, int nsrc, void *out, size_t numel, int dtype, hipStream_t stream,
                 const tccl_launch_cfg *cfg)
@@ -89,8 +179,17 @@ int sum_streams(const void *const *srcs, int nsrc, void *out, size_t numel, int 
     if (numel == 0) return TCCL_OK;
 
     const size_t nvec = numel * static_cast<size_t>(esize) / kVecBytes;
-    const Shape sh = resolve_shape(cfg, nvec, nsrc, 1);
     const char *const *s = reinterpret_cast<const char *const *>(srcs);
+    const int flags = cfg ? cfg->flags : 0;
+    const bool phased = (flags & TCCL_CFG_PHASED) ||
+                        (!(flags & TCCL_CFG_STREAMING) && nvec * kVecBytes >= phased_min_bytes(nsrc));
+    if (phased) {
+        hipError_t pe = (dtype == TCCL_BF16)
+                            ? launch_phased_nsrc<Bf16Sum>(s, nsrc, static_cast<char *>(out), numel, cfg, stream)
+                            : launch_phased_nsrc<F32Sum>(s, nsrc, static_cast<char *>(out), numel, cfg, stream);
+        return hip_code(pe);
+    }
+    const Shape sh = resolve_shape(cfg, nvec, nsrc, 1);
     hipError_t e = (dtype == TCCL_BF16) ? launch_sum_nsrc<Bf16Sum>(s, nsrc, static_cast<char *>(out), numel, sh, stream)
                                         : launch_sum_nsrc<F32Sum>(s, nsrc, static_cast<char *>(out), numel, sh, stream);
     return hip_code(e);

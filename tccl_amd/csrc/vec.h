@@ -219,6 +219,135 @@ __device__ __forceinline__ void sum_range(const char *const (&src)[NSRC], char *
     }
 }
 
+// ---------------------------------------------------------------------------------
+// Phased tiles.  HBM serves reads and writes over one data bus and loses time on every
+// turn-around, so a kernel that interleaves its output stores with its input loads runs
+// well below the sum of a pure read pass and a pure write pass.  A phased workgroup owns
+// one contiguous tile: it reads and reduces the whole tile into registers first
+// (K iterations of U vectors per lane) and only then writes the tile's results, back to
+// back.  When all workgroups of a launch are resident at once and run at the same pace,
+// the launch as a whole turns into one long read phase followed by one write burst.
+//
+// Tiles are addressed through buffer descriptors whose size is the exact number of valid
+// bytes left in the tile: loads beyond the end return zero and stores beyond the end are
+// dropped by the hardware, so a partial tile needs no branches.
+
+constexpr int kPhasedBlock = 256; // lanes per workgroup
+constexpr int kPhasedVecs = 32;   // result vectors a lane holds before it writes (128 VGPRs)
+constexpr int kAuxLoadStream = 2;   // cache policy of the loads: nt (stream through L2)
+constexpr int kAuxStoreStream = 16; // cache policy of the stores: sc1 (write through to memory)
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const char *tile_start, uint32_t valid_bytes)
+{
+    // stride 0 (raw buffer), 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(tile_start), 0, static_cast<int>(valid_bytes),
+                                             0x00020000);
+}
+
+// Vectors per lane per iteration for a given number of sources: keeps 12 to 16 loads of
+// 16 bytes in flight per lane.
+template <int NSRC>
+struct PhasedUnroll {
+    static constexpr int value = NSRC <= 2 ? 8 : (NSRC <= 4 ? 4 : 2);
+    static constexpr int kmax = kPhasedVecs / value; // most iterations per tile
+};
+
+// One tile: sources [tile_off, tile_off + valid) -> destinations, `kcount` <= KMAX
+// iterations of kPhasedBlock * U vectors.  valid is a multiple of 16 (may be 0).
+template <class Sum, int NSRC, int NDST, int U, int KMAX>
+__device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], char *const (&dst)[NDST],
+                                                size_t tile_off, uint32_t valid_bytes, int kcount)
+{
+    __amdgpu_buffer_rsrc_t rs[NSRC];
+#pragma unroll
+    for (int s = 0; s < NSRC; ++s) rs[s] = tile_rsrc(src[s] + tile_off, valid_bytes);
+    constexpr uint32_t span_bytes = kPhasedBlock * U * kVecBytes;
+    const uint32_t lane_off = threadIdx.x * kVecBytes;
+
+    u32x4 r[KMAX][U];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        if (k < kcount) {
+            u32x4 v[U][NSRC];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int s = 0; s < NSRC; ++s)
+                    v[u][s] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rs[s], k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxLoadStream);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                Sum acc;
+                acc.zero();
+#pragma unroll
+                for (int s = 0; s < NSRC; ++s) acc.add(v[u][s]);
+                r[k][u] = acc.result();
+            }
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < NDST; ++d) {
+        const __amdgpu_buffer_rsrc_t rd = tile_rsrc(dst[d] + tile_off, valid_bytes);
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) {
+            if (k < kcount) {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    __builtin_amdgcn_raw_buffer_store_b128(
+                        r[k][u], rd, k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxStoreStream);
+            }
+        }
+    }
+}
+
+// Same walk for a plain copy of one source into NDST destinations.
+template <int NDST, int U, int KMAX>
+__device__ __forceinline__ void copy_tile_phased(const char *src, char *const (&dst)[NDST], size_t tile_off,
+                                                 uint32_t valid_bytes, int kcount)
+{
+    const __amdgpu_buffer_rsrc_t rs = tile_rsrc(src + tile_off, valid_bytes);
+    constexpr uint32_t span_bytes = kPhasedBlock * U * kVecBytes;
+    const uint32_t lane_off = threadIdx.x * kVecBytes;
+    u32x4 r[KMAX][U];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        if (k < kcount) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                r[k][u] = __builtin_amdgcn_raw_buffer_load_b128(
+                    rs, k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxLoadStream);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < NDST; ++d) {
+        const __amdgpu_buffer_rsrc_t rd = tile_rsrc(dst[d] + tile_off, valid_bytes);
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) {
+            if (k < kcount) {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    __builtin_amdgcn_raw_buffer_store_b128(
+                        r[k][u], rd, k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxStoreStream);
+            }
+        }
+    }
+}
+
+// The ragged tail: elements [first, numel), fewer than one vector, one lane each.
+template <class Sum, int NSRC, int NDST>
+__device__ __forceinline__ void sum_tail(const char *const (&src)[NSRC], char *const (&dst)[NDST], size_t first,
+                                         size_t numel)
+{
+    const size_t i = first + threadIdx.x;
+    if (i < numel) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NSRC; ++s) acc = acc + Sum::widen(src[s], i);
+#pragma unroll
+        for (int d = 0; d < NDST; ++d) Sum::narrow(dst[d], i, acc);
+    }
+}
+
 // Copy one source into NDST destinations over [0, nvec) vectors; same tiling as sum_range.
 template <int NDST, int UNROLL, bool NTL, bool NTS>
 __device__ __forceinline__ void copy_range(const char *src, char *const (&dst)[NDST], size_t nvec,

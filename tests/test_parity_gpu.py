@@ -109,6 +109,48 @@ def test_all_reduce_every_launch_shape(block, unroll, flags, _gpu_hygiene, c_ora
     assert_bit_equal(tccl_amd.one_shot_all_reduce(g3.tensor(0), cfg=cfg), oracle_sum(c_oracle, small), "W=3")
 
 
+@pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+def test_all_reduce_phased_kernel_forced(world, maker, _gpu_hygiene, c_oracle):
+    """The read-then-write kernel that large inputs take, forced onto small inputs so that
+    partial tiles, several launches per call, every tile length and ragged tails are all
+    exercised against the oracle."""
+    per_vec = 8 if maker is seeded_randn else 4
+    numel = per_vec * 100_003 + 3                      # not a whole number of vectors
+    bufs = maker(world, numel + per_vec)
+    g = upload(_gpu_hygiene, bufs)
+    want = oracle_sum(c_oracle, [b[:numel].contiguous() for b in bufs])
+    dt = _lib.TCCL_BF16 if bufs[0].dtype == torch.bfloat16 else _lib.TCCL_F32
+    lib = tccl_amd.load_library()
+    for tile_iters, grid in ((0, 0), (1, 0), (1, 7), (2, 3), (3, 16), (4, 512), (5, 1), (8, 2), (16, 4), (16, 1)):
+        cfg = tccl_amd.LaunchCfg(grid=grid, tile_iters=tile_iters, flags=_lib.CFG_PHASED)
+        out = torch.full((numel + 16,), 55.0, dtype=bufs[0].dtype, device=DEV)
+        rc = lib.tccl_all_reduce_sum_ex(g.ptr_array, world, out.data_ptr(), numel, dt, stream(), ctypes.byref(cfg))
+        assert rc == 0
+        assert_bit_equal(out[:numel], want, f"W={world} K={tile_iters} grid={grid}")
+        assert out[numel:].eq(55.0).all().item(), "wrote past the end"
+    # sizes below one vector and exactly one tile
+    for n in (0, 1, per_vec - 1, per_vec, 256 * per_vec * 2, 256 * per_vec * 2 * 16 + 1):
+        cfg = tccl_amd.LaunchCfg(flags=_lib.CFG_PHASED)
+        out = torch.full((n + 16,), 55.0, dtype=bufs[0].dtype, device=DEV)
+        assert lib.tccl_all_reduce_sum_ex(g.ptr_array, world, out.data_ptr(), n, dt, stream(), ctypes.byref(cfg)) == 0
+        w = oracle_sum(c_oracle, [b[:n].contiguous() for b in bufs]) if n else bufs[0][:0]
+        assert_bit_equal(out[:n], w, f"W={world} n={n}")
+        assert out[n:].eq(55.0).all().item()
+
+
+def test_phased_and_streaming_kernels_agree_at_headline_size(_gpu_hygiene, c_oracle):
+    """W=8 x 64 MiB bf16: default dispatch (phased), forced streaming, and the oracle."""
+    n = (64 << 20) // 2
+    bufs = seeded_randn(8, n)
+    g = upload(_gpu_hygiene, bufs)
+    want = oracle_sum(c_oracle, bufs)
+    assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0)), want, "default")
+    for flags in (_lib.CFG_STREAMING | 3, _lib.CFG_PHASED):
+        cfg = tccl_amd.LaunchCfg(flags=flags)
+        assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0), cfg=cfg), want, f"flags={flags}")
+
+
 def test_all_reduce_order_and_single_rounding(_gpu_hygiene):
     """fp32 accumulation in rank order: [2^24, 1 x6, -2^24] -> 0; ones first -> 6;
     1 + 2^-8 + 2^-8 -> 1 + 2^-7 (a bf16-stepwise sum would give 1)."""
@@ -290,6 +332,20 @@ def test_tree_reduce_step(children, maker, in_place, _gpu_hygiene, c_oracle):
     assert_bit_equal(dst, want, f"children={children}")
     assert_bit_equal(d0, c0, "child0 untouched")
     assert_bit_equal(d1, c1, "child1 untouched")
+
+
+def test_tree_reduce_step_large_in_place(_gpu_hygiene, c_oracle):
+    """128 MiB half of a 256 MiB bf16 buffer, own + two children, stored over own."""
+    numel = 67_108_864
+    torch.manual_seed(1)
+    base = torch.randn(numel, dtype=torch.bfloat16)
+    own, c0, c1 = base, base.roll(12_345_677), base.roll(-7_654_321)
+    want = oracle_sum(c_oracle, [c0, c1, own])
+    d_own, d0, d1 = own.to(DEV), c0.to(DEV), c1.to(DEV)
+    rc = tccl_amd.load_library().tccl_tree_reduce_step(d_own.data_ptr(), d0.data_ptr(), d1.data_ptr(),
+                                                       d_own.data_ptr(), numel, _lib.TCCL_BF16, stream())
+    assert rc == 0
+    assert_bit_equal(d_own, want, "in place, large")
 
 
 @pytest.mark.parametrize("two", [False, True])
