@@ -69,7 +69,8 @@ typedef struct {
 #define TCCL_CFG_STREAMING 16        /* force the grid-stride kernel (stores interleaved with loads) */
 #define TCCL_CFG_PHASED 32           /* force the phased kernel (each workgroup reads its whole tile,
                                         then writes it); there `grid` = workgroups per launch and
-                                        `tile_iters` = iterations per tile (1..16), block/unroll unused */
+                                        `tile_iters` = iterations per tile, `unroll` = vectors per lane per
+                                        iteration (iterations * unroll <= 32), block unused */
 
 int tccl_abi_version(void);
 const char *tccl_error_string(int code);

@@ -78,42 +78,41 @@ static hipError_t launch_sum_nsrc(const char *const *srcs, int nsrc, char *out, 
 // ---------------------------------------------------------------------------------
 // Phased variant: one tile per workgroup, all of a launch's workgroups resident at once.
 
-template <class Sum, int NSRC>
+template <class Sum, int NSRC, int U, bool FULL>
 __global__ void __launch_bounds__(kPhasedBlock)
 sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_t tail_first, size_t numel)
 {
-    constexpr int U = PhasedUnroll<NSRC>::value;
-    constexpr int KMAX = PhasedUnroll<NSRC>::kmax;
+    constexpr int KMAX = kPhasedVecs / U;
     const size_t tile_bytes = static_cast<size_t>(kcount) * (kPhasedBlock * U * kVecBytes);
     const size_t off = blockIdx.x * tile_bytes;
     const size_t left = bytes > off ? bytes - off : 0;
     const uint32_t valid = static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes);
     char *const dst[1] = {out};
-    sum_tile_phased<Sum, NSRC, 1, U, KMAX>(src.p, dst, off, valid, kcount);
+    sum_tile_phased<Sum, NSRC, 1, U, KMAX, FULL>(src.p, dst, off, valid, kcount);
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
 }
 
-template <class Sum, int NSRC>
-static hipError_t launch_phased(const char *const *srcs, char *out, size_t numel, const tccl_launch_cfg *cfg,
-                                hipStream_t stream)
+template <class Sum, int NSRC, int U>
+static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t numel, const tccl_launch_cfg *cfg,
+                                  hipStream_t stream)
 {
-    constexpr int U = PhasedUnroll<NSRC>::value;
-    constexpr size_t kPhasedKMax = PhasedUnroll<NSRC>::kmax;
+    constexpr size_t kmax = kPhasedVecs / U;
     constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
     constexpr size_t span = static_cast<size_t>(kPhasedBlock) * U; // vectors per iteration
     const size_t nvec = numel / per_vec;
     size_t wgs = (cfg && cfg->grid > 0) ? static_cast<size_t>(cfg->grid) : static_cast<size_t>(compute_units()) * 2;
     size_t kcount;
     if (cfg && cfg->tile_iters > 0) {
-        kcount = static_cast<size_t>(cfg->tile_iters) > kPhasedKMax ? kPhasedKMax : cfg->tile_iters;
+        kcount = static_cast<size_t>(cfg->tile_iters) > kmax ? kmax : cfg->tile_iters;
     } else {
         // Fewest launches that fit, then the smallest tile that covers a launch's share
         // with `wgs` workgroups, so that every launch is one full, even wave of workgroups.
-        const size_t launches = (nvec + wgs * span * kPhasedKMax - 1) / (wgs * span * kPhasedKMax);
-        const size_t per_launch = (nvec + (launches ? launches : 1) - 1) / (launches ? launches : 1);
+        size_t launches = (nvec + wgs * span * kmax - 1) / (wgs * span * kmax);
+        if (launches == 0) launches = 1;
+        const size_t per_launch = (nvec + launches - 1) / launches;
         kcount = (per_launch + wgs * span - 1) / (wgs * span);
         if (kcount < 1) kcount = 1;
-        if (kcount > kPhasedKMax) kcount = kPhasedKMax;
+        if (kcount > kmax) kcount = kmax;
     }
     const size_t tile_vec = kcount * span;
     const size_t slice_vec = wgs * tile_vec;
@@ -130,14 +129,28 @@ static hipError_t launch_phased(const char *const *srcs, char *out, size_t numel
         // the tail's element indices are relative to this launch's base pointers
         const size_t rel_first = last ? tail_first - off * per_vec : 0;
         const size_t rel_numel = last ? numel - off * per_vec : 0;
-        hipLaunchKernelGGL((sum_phased_kernel<Sum, NSRC>), dim3(static_cast<unsigned>(grid)), dim3(kPhasedBlock), 0,
-                           stream, t, out + off * kVecBytes, n * kVecBytes, static_cast<int>(kcount), rel_first,
-                           rel_numel);
+        if (kcount == kmax)
+            hipLaunchKernelGGL((sum_phased_kernel<Sum, NSRC, U, true>), dim3(static_cast<unsigned>(grid)),
+                               dim3(kPhasedBlock), 0, stream, t, out + off * kVecBytes, n * kVecBytes,
+                               static_cast<int>(kcount), rel_first, rel_numel);
+        else
+            hipLaunchKernelGGL((sum_phased_kernel<Sum, NSRC, U, false>), dim3(static_cast<unsigned>(grid)),
+                               dim3(kPhasedBlock), 0, stream, t, out + off * kVecBytes, n * kVecBytes,
+                               static_cast<int>(kcount), rel_first, rel_numel);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         off += n;
     } while (off < nvec);
     return hipSuccess;
+}
+
+template <class Sum, int NSRC>
+static hipError_t launch_phased(const char *const *srcs, char *out, size_t numel, const tccl_launch_cfg *cfg,
+                                hipStream_t stream)
+{
+    if (cfg && cfg->unroll == PhasedUnroll<NSRC>::alt)
+        return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::alt>(srcs, out, numel, cfg, stream);
+    return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::value>(srcs, out, numel, cfg, stream);
 }
 
 template <class Sum>
@@ -157,13 +170,10 @@ static hipError_t launch_phased_nsrc(const char *const *srcs, int nsrc, char *ou
     }
 }
 
-// Inputs of at least this many output bytes take the phased kernel: below it a launch
-// cannot give every compute unit two tiles of at least two iterations.
-static size_t phased_min_bytes(int nsrc)
-{
-    const int u = nsrc <= 2 ? 8 : (nsrc <= 4 ? 4 : 2);
-    return static_cast<size_t>(compute_units()) * 2 * kPhasedBlock * u * kVecBytes * 2;
-}
+// Inputs with at least this many output bytes take the phased kernel; smaller ones finish
+// in a few microseconds either way and take the grid-stride kernel, whose launch shape
+// adapts to tiny inputs.
+static size_t phased_min_bytes(int) { return static_cast<size_t>(4) << 20; }
 
 // Sum `nsrc` already-offset source pointers into `out`.  Shared by the three entry points.
 int sum_streams(const void *const *srcs, int nsrc, void *out, size_t numel, int dtype, hipStream_t stream,

@@ -11,63 +11,80 @@ struct JobTable {
     tccl_node_job job[TCCL_MAX_JOBS];
 };
 
-// One node step over its element range.  blockIdx.y selects the job; the workgroups of a
-// job walk its range one pipelining chunk (tile) at a time, so a chunk is read, reduced
-// and written by a single workgroup, the way one message of the tree pipeline would be.
-template <class Sum, int NSRC, int NDST>
-__device__ __forceinline__ void run_reduce(const tccl_node_job &j, const char *const (&src)[NSRC], int tile_iters)
-{
-    if constexpr (NDST == 2) {
-        char *const dst[2] = {static_cast<char *>(j.dst[0]), static_cast<char *>(j.dst[1])};
-        sum_range<Sum, NSRC, 2, 2, false, false>(src, dst, j.numel, tile_iters, false);
-    } else {
-        char *const dst[1] = {static_cast<char *>(j.dst[0])};
-        sum_range<Sum, NSRC, 1, 2, false, false>(src, dst, j.numel, tile_iters, false);
-    }
-}
+// One node step over its element range.  blockIdx.y selects the job; workgroup x of a job
+// takes tile x, x + gridDim.x, ...  A tile is one pipelining chunk (or a 128 KiB piece of
+// it when chunks are larger): its sources are read and reduced into registers, then the
+// result is written, the way one message of the tree pipeline would be received, reduced
+// and forwarded.
+constexpr int kLevelU = 2;
+constexpr int kLevelKMax = kPhasedVecs / kLevelU;
 
-template <class Sum, int NDST>
-__device__ __forceinline__ void run_job(const tccl_node_job &j, int tile_iters)
+template <class Sum, int NDST, bool FULL>
+__device__ __forceinline__ void run_tile(const tccl_node_job &j, char *const (&dst)[NDST], size_t off, uint32_t valid,
+                                         int kcount)
 {
     const char *c0 = static_cast<const char *>(j.src[0]);
     const char *c1 = static_cast<const char *>(j.src[1]);
     const char *own = static_cast<const char *>(j.src[2]);
     if (j.is_copy) {
-        const size_t nvec = j.numel * Sum::kElemBytes / kVecBytes;
-        if constexpr (NDST == 2) {
-            char *const dst[2] = {static_cast<char *>(j.dst[0]), static_cast<char *>(j.dst[1])};
-            copy_range<2, 2, false, false>(c0, dst, nvec, tile_iters, false);
-        } else {
-            char *const dst[1] = {static_cast<char *>(j.dst[0])};
-            copy_range<1, 2, false, false>(c0, dst, nvec, tile_iters, false);
-        }
+        copy_tile_phased<NDST, kLevelU, kLevelKMax>(c0, dst, off, valid, kcount);
     } else if (c0 != nullptr && c1 != nullptr) {
         const char *const src[3] = {c0, c1, own};
-        run_reduce<Sum, 3, NDST>(j, src, tile_iters);
-    } else if (c0 != nullptr) {
-        const char *const src[2] = {c0, own};
-        run_reduce<Sum, 2, NDST>(j, src, tile_iters);
-    } else if (c1 != nullptr) {
-        const char *const src[2] = {c1, own};
-        run_reduce<Sum, 2, NDST>(j, src, tile_iters);
+        sum_tile_phased<Sum, 3, NDST, kLevelU, kLevelKMax, FULL>(src, dst, off, valid, kcount);
+    } else if (c0 != nullptr || c1 != nullptr) {
+        const char *const src[2] = {c0 != nullptr ? c0 : c1, own};
+        sum_tile_phased<Sum, 2, NDST, kLevelU, kLevelKMax, FULL>(src, dst, off, valid, kcount);
     } else {
         const char *const src[1] = {own};
-        run_reduce<Sum, 1, NDST>(j, src, tile_iters);
+        sum_tile_phased<Sum, 1, NDST, kLevelU, kLevelKMax, FULL>(src, dst, off, valid, kcount);
     }
 }
 
-template <class Sum>
-__global__ void __launch_bounds__(kMaxBlock) tree_level_kernel(JobTable jobs, int tile_iters)
+template <class Sum, int NDST>
+__device__ __forceinline__ void run_tail(const tccl_node_job &j, char *const (&dst)[NDST], size_t first)
+{
+    const char *c0 = static_cast<const char *>(j.src[0]);
+    const char *c1 = static_cast<const char *>(j.src[1]);
+    const char *own = static_cast<const char *>(j.src[2]);
+    if (c0 != nullptr && c1 != nullptr) {
+        const char *const src[3] = {c0, c1, own};
+        sum_tail<Sum, 3, NDST>(src, dst, first, j.numel);
+    } else if (c0 != nullptr || c1 != nullptr) {
+        const char *const src[2] = {c0 != nullptr ? c0 : c1, own};
+        sum_tail<Sum, 2, NDST>(src, dst, first, j.numel);
+    } else {
+        const char *const src[1] = {own};
+        sum_tail<Sum, 1, NDST>(src, dst, first, j.numel);
+    }
+}
+
+template <class Sum, int NDST, bool FULL>
+__device__ __forceinline__ void run_job(const tccl_node_job &j, int kcount)
+{
+    char *dst[NDST];
+#pragma unroll
+    for (int d = 0; d < NDST; ++d) dst[d] = static_cast<char *>(j.dst[d]);
+    char *const(&cdst)[NDST] = dst;
+    constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
+    const size_t bytes = j.numel / per_vec * kVecBytes;
+    const size_t tile_bytes = static_cast<size_t>(kcount) * (kPhasedBlock * kLevelU * kVecBytes);
+    for (size_t off = blockIdx.x * tile_bytes; off < bytes; off += gridDim.x * tile_bytes) {
+        const size_t left = bytes - off;
+        run_tile<Sum, NDST, FULL>(j, cdst, off, static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes), kcount);
+    }
+    // ragged tail of a reduce step (copy steps are whole vectors)
+    if (blockIdx.x == 0 && !j.is_copy && j.numel % per_vec != 0) run_tail<Sum, NDST>(j, cdst, j.numel / per_vec * per_vec);
+}
+
+template <class Sum, bool FULL>
+__global__ void __launch_bounds__(kPhasedBlock) tree_level_kernel(JobTable jobs, int kcount)
 {
     const tccl_node_job &j = jobs.job[blockIdx.y];
     if (j.dst[1] != nullptr)
-        run_job<Sum, 2>(j, tile_iters);
+        run_job<Sum, 2, FULL>(j, kcount);
     else
-        run_job<Sum, 1>(j, tile_iters);
+        run_job<Sum, 1, FULL>(j, kcount);
 }
-
-constexpr int kLevelBlock = 256;
-constexpr int kLevelUnroll = 2; // matches the UNROLL used in run_reduce / run_job
 
 int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_elems, hipStream_t stream)
 {
@@ -76,10 +93,10 @@ int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_e
     if (njobs == 0) return TCCL_OK;
     const size_t per_vec = kVecBytes / esize;
     if (chunk_elems == 0) chunk_elems = (128u * 1024u) / esize;
-    const size_t span = static_cast<size_t>(kLevelBlock) * kLevelUnroll; // vectors per iteration
-    size_t tile_iters = (chunk_elems / per_vec + span - 1) / span;
-    if (tile_iters < 1) tile_iters = 1;
-    if (tile_iters > (1u << 20)) return TCCL_EINVAL;
+    const size_t span = static_cast<size_t>(kPhasedBlock) * kLevelU; // vectors per iteration
+    size_t kcount = (chunk_elems / per_vec + span - 1) / span;
+    if (kcount < 1) kcount = 1;
+    if (kcount > kLevelKMax) kcount = kLevelKMax; // larger chunks are walked in 128 KiB pieces
 
     JobTable t = {};
     size_t max_tiles = 0;
@@ -93,20 +110,25 @@ int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_e
         if (j.is_copy && (j.numel % per_vec) != 0) return TCCL_EALIGN;
         t.job[i] = j;
         const size_t nvec = j.numel / per_vec;
-        const size_t tiles = (nvec + span * tile_iters - 1) / (span * tile_iters);
+        const size_t tiles = (nvec + span * kcount - 1) / (span * kcount);
         if (tiles > max_tiles) max_tiles = tiles;
     }
     if (max_tiles == 0) max_tiles = 1; // ragged tails only
-    // Enough workgroups over all jobs to fill the chip about eight deep, no more than one
-    // per chunk.
-    size_t want = (static_cast<size_t>(compute_units()) * 8 + njobs - 1) / njobs;
-    const unsigned gx = static_cast<unsigned>(max_tiles < want ? max_tiles : want);
-    if (dtype == TCCL_BF16)
-        hipLaunchKernelGGL(tree_level_kernel<Bf16Sum>, dim3(gx, njobs), dim3(kLevelBlock), 0, stream, t,
-                           static_cast<int>(tile_iters));
-    else
-        hipLaunchKernelGGL(tree_level_kernel<F32Sum>, dim3(gx, njobs), dim3(kLevelBlock), 0, stream, t,
-                           static_cast<int>(tile_iters));
+    if (max_tiles > 0x7FFFFFFFu) max_tiles = 0x7FFFFFFFu;
+    const dim3 grid(static_cast<unsigned>(max_tiles), njobs);
+    const int kc = static_cast<int>(kcount);
+    const bool full = kcount == static_cast<size_t>(kLevelKMax);
+    if (dtype == TCCL_BF16) {
+        if (full)
+            hipLaunchKernelGGL((tree_level_kernel<Bf16Sum, true>), grid, dim3(kPhasedBlock), 0, stream, t, kc);
+        else
+            hipLaunchKernelGGL((tree_level_kernel<Bf16Sum, false>), grid, dim3(kPhasedBlock), 0, stream, t, kc);
+    } else {
+        if (full)
+            hipLaunchKernelGGL((tree_level_kernel<F32Sum, true>), grid, dim3(kPhasedBlock), 0, stream, t, kc);
+        else
+            hipLaunchKernelGGL((tree_level_kernel<F32Sum, false>), grid, dim3(kPhasedBlock), 0, stream, t, kc);
+    }
     return hip_code(hipGetLastError());
 }
 

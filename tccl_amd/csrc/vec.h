@@ -244,17 +244,19 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const char *tile_sta
                                              0x00020000);
 }
 
-// Vectors per lane per iteration for a given number of sources: keeps 12 to 16 loads of
-// 16 bytes in flight per lane.
+// Vectors per lane per iteration for a given number of sources (two candidates each,
+// the first is the default).
 template <int NSRC>
 struct PhasedUnroll {
-    static constexpr int value = NSRC <= 2 ? 8 : (NSRC <= 4 ? 4 : 2);
-    static constexpr int kmax = kPhasedVecs / value; // most iterations per tile
+    static constexpr int value = NSRC <= 2 ? 4 : (NSRC <= 4 ? 2 : 1);
+    static constexpr int alt = value * 2;
 };
 
 // One tile: sources [tile_off, tile_off + valid) -> destinations, `kcount` <= KMAX
 // iterations of kPhasedBlock * U vectors.  valid is a multiple of 16 (may be 0).
-template <class Sum, int NSRC, int NDST, int U, int KMAX>
+// FULL = the tile has exactly KMAX iterations: straight-line code, which lets the
+// compiler start the loads of the next iteration before the adds of this one.
+template <class Sum, int NSRC, int NDST, int U, int KMAX, bool FULL>
 __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], char *const (&dst)[NDST],
                                                 size_t tile_off, uint32_t valid_bytes, int kcount)
 {
@@ -267,7 +269,7 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
     u32x4 r[KMAX][U];
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
-        if (k < kcount) {
+        if (FULL || k < kcount) {
             u32x4 v[U][NSRC];
 #pragma unroll
             for (int u = 0; u < U; ++u)
@@ -290,7 +292,7 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
         const __amdgpu_buffer_rsrc_t rd = tile_rsrc(dst[d] + tile_off, valid_bytes);
 #pragma unroll
         for (int k = 0; k < KMAX; ++k) {
-            if (k < kcount) {
+            if (FULL || k < kcount) {
 #pragma unroll
                 for (int u = 0; u < U; ++u)
                     __builtin_amdgcn_raw_buffer_store_b128(
