@@ -30,9 +30,11 @@ WORLD = 8
 BYTES_PER_BUF = 64 << 20
 LAT_BYTES_PER_BUF = 1 << 20
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
-# scaled by what the same counters read for a plain copy of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs of this script
+# (FETCH_SIZE 262,353.78 KiB and WRITE_SIZE 65,536.00 KiB per dispatch), each scaled by what
+# the same counter reads for the 256 MiB plain copy of --calibrate-copy (factors 1.99959 and
+# 1.00000): 524,601 KiB fetched + 65,536 KiB written.
+MEASURED_TRAFFIC_BYTES = 604_300_375
 
 
 def parse_args():
@@ -42,6 +44,9 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     p.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU work budget for the baseline leg")
+    p.add_argument("--calibrate-copy", action="store_true",
+                   help="also run 20 plain copies of 256 MiB (tccl_tree_copy_step), so that a rocprofv3 --pmc "
+                        "run of this command holds a kernel of known traffic to scale the counters by")
     p.add_argument("--sweep", action="store_true",
                    help="also time every op and size of the sweep; written to stderr as JSON lines")
     return p.parse_args()
@@ -197,7 +202,7 @@ def main():
             "unit": "GB/s",
             "frac": round(gbs_dev / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES,
-            "kernel": "tccl::sum_kernel<Bf16Sum, 8, ...>",
+            "kernel": "tccl::sum_phased_kernel<Bf16Sum, 8, 1, true>",
             "avg_launch_us": round(dev_ms * 1e3, 2),
             "algorithmic_bytes": algo_bytes,
         },
@@ -222,6 +227,17 @@ def main():
             "gpu_matches_cpu_bitwise": bool(same),
         }
         del bufs_cpu
+
+    if args.calibrate_copy:
+        nbytes = 256 << 20
+        src = torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device=device)
+        dst = torch.empty_like(src)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for _ in range(20):
+            assert lib.tccl_tree_copy_step(src.data_ptr(), dst.data_ptr(), None, nbytes, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+        del src, dst
 
     if args.sweep:
         run_sweep(torch, tccl_amd, lib, device)
