@@ -94,6 +94,49 @@ def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, 
     return output
 
 
+def two_shot_all_reduce(tensor: torch.Tensor) -> torch.Tensor:
+    """All-reduce as reduce-scatter followed by all-gather (the composition the reference's
+    slides name for large messages: "can be combined with reduce-scatter for all-reduce").
+
+    Every rank reduces its own 1/W share (one ``tccl_reduce_scatter_sum`` launch per rank),
+    the shares form a symmetric group of their own, and the output is their all-gather.  The
+    result is bit-identical to ``one_shot_all_reduce``: every element is still the fp32 sum
+    over the ranks in rank order.  Same precondition as the reduce-scatter
+    (triton_reduce_scatter.py:101-104).  On several GPUs this moves (W-1)/W of a buffer per
+    direction over the links instead of (W-1) whole buffers."""
+    dtype = _sum_dtype(tensor)
+    symm = rendezvous(tensor)
+    world = symm.world_size
+    assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
+    per_rank = tensor.numel() // world
+    lib = _lib.load()
+    stream = _stream()
+    shares = torch.empty((world, per_rank), dtype=tensor.dtype, device=tensor.device)
+    for r in range(world):
+        rc = lib.tccl_reduce_scatter_sum(symm.buffer_ptrs_host, world, r, shares[r].data_ptr(), tensor.numel(),
+                                         dtype, stream)
+        _lib.check("tccl_reduce_scatter_sum", rc)
+    share_ptrs = _lib.ptr_array([int(shares[r].data_ptr()) for r in range(world)])
+    output = torch.empty_like(tensor)
+    rc = lib.tccl_all_gather(share_ptrs, world, output.data_ptr(), per_rank * tensor.element_size(), stream)
+    _lib.check("tccl_all_gather", rc)
+    return output
+
+
+def all_reduce(tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
+    """All-reduce by the named algorithm: ``"one_shot"``, ``"two_shot"``, ``"double_tree"`` or
+    ``"auto"``.  With every buffer in the same HBM the one-shot kernel moves the fewest bytes
+    ((W+1)N against (W+3)N for two-shot and more for the tree), so ``"auto"`` is one-shot at
+    every size; the other two exist for what they model across GPUs."""
+    if algorithm in ("auto", "one_shot"):
+        return one_shot_all_reduce(tensor)
+    if algorithm == "two_shot":
+        return two_shot_all_reduce(tensor)
+    if algorithm == "double_tree":
+        return double_tree_all_reduce(tensor)
+    raise ValueError(f"unknown all-reduce algorithm {algorithm!r}")
+
+
 def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tensor,
                      chunk_elems: int) -> List[torch.Tensor]:
     outputs = [torch.empty_like(like) for _ in range(group.world_size)]

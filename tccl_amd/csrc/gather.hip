@@ -105,7 +105,7 @@ extern "C" int tccl_all_gather_ex(const void *const *bufs, int world, void *out,
     }
     if (bytes_per_rank == 0) return TCCL_OK;
     const size_t row_vecs = bytes_per_rank / kVecBytes;
-    const Shape sh = resolve_shape(cfg, row_vecs, 1, world);
+    const Shape sh = resolve_shape(cfg, row_vecs, 1, world, true);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char *o = static_cast<char *>(out);
     hipError_t e;
@@ -128,7 +128,7 @@ extern "C" int tccl_tree_copy_step(const void *src, void *dst0, void *dst1, size
     if (bytes % kVecBytes != 0 || !aligned16(src) || !aligned16(dst0) || !aligned16(dst1)) return TCCL_EALIGN;
     if (bytes == 0) return TCCL_OK;
     const size_t nvec = bytes / kVecBytes;
-    const Shape sh = resolve_shape(nullptr, nvec, 1, 1);
+    const Shape sh = resolve_shape(nullptr, nvec, 1, 1, true);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const char *in = static_cast<const char *>(src);
     hipError_t e = dst1 ? launch_copy_unroll<2>(in, static_cast<char *>(dst0), static_cast<char *>(dst1), nvec, sh, s)

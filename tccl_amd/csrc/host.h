@@ -36,6 +36,8 @@ struct Shape {
 //   nvec      -- 16-byte vectors of output the launch produces (per row for the gather)
 //   nsrc      -- source streams read per output vector
 //   rows      -- independent rows sharing the grid's y dimension (gather), else 1
-Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows);
+//   is_copy   -- a pure copy: large ones default to streaming (nt) stores, which on this
+//                memory system is worth 20 % once the output no longer fits the caches
+Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows, bool is_copy = false);
 
 } // namespace tccl

@@ -22,7 +22,7 @@ int compute_units()
     return cu;
 }
 
-Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows)
+Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows, bool is_copy)
 {
     tccl_launch_cfg c = {};
     if (cfg) c = *cfg;
@@ -36,7 +36,7 @@ Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows)
     if (c.unroll == 1 || c.unroll == 2 || c.unroll == 4) {
         sh.unroll = c.unroll;
     } else {
-        int u = 8 / nsrc;
+        int u = is_copy ? 2 : 8 / nsrc;
         u = u >= 4 ? 4 : (u >= 2 ? 2 : 1);
         while (u > 1 && nvec * rows / (static_cast<size_t>(sh.block) * u) < static_cast<size_t>(cus) * 2) u /= 2;
         sh.unroll = u;
@@ -57,6 +57,8 @@ Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows)
     } else {
         sh.nt_load = (flags & TCCL_CFG_NONTEMPORAL_LOAD) != 0;
         sh.nt_store = (flags & TCCL_CFG_NONTEMPORAL_STORE) != 0;
+        const bool unspecified = (flags & (TCCL_CFG_NONTEMPORAL_LOAD | TCCL_CFG_NONTEMPORAL_STORE)) == 0;
+        if (is_copy && unspecified && nvec * rows * kVecBytes >= (static_cast<size_t>(8) << 20)) sh.nt_store = true;
     }
 
     // Workgroups: enough to keep every compute unit at full wave occupancy

@@ -1,0 +1,76 @@
+"""Size sweep in the shape of the reference's ``__main__`` benchmarks.
+
+The reference halves the message size from 256 Mi elements down to 2,048 and prints one
+line per size, ``"<name> <bytes> <rate> MB/s"`` (triton_reduce_scatter.py:213-240,
+triton_all_gather.py:177-204, triton_double_tree_allreduce.py:412-438); its "MB/s" is
+really bytes / ms / 1e6 = GB/s of *input bytes per rank*, timed over 10 calls with no
+warm-up.  This harness prints the same columns with the unit fixed (GB/s of input bytes per
+rank, as the reference counts them) plus the algorithmic HBM GB/s, after a warm-up, timed
+with HIP events on the launch stream.
+
+    python -m tccl_amd.harness all_reduce|reduce_scatter|all_gather|double_tree [--world 8] [--max-elems N]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import sys
+
+REPS = 10          # as in the reference
+
+
+def main(argv=None) -> int:
+    p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    p.add_argument("op", choices=["all_reduce", "reduce_scatter", "all_gather", "double_tree", "two_shot"])
+    p.add_argument("--world", type=int, default=8)
+    p.add_argument("--max-elems", type=int, default=256 * 1024 * 1024 // 2,
+                   help="largest element count per rank (bf16); halved down to 2,048")
+    args = p.parse_args(argv)
+
+    import torch
+    import tccl_amd
+    lib = tccl_amd.load_library()
+    world = args.world
+    group = tccl_amd.empty_world(world, args.max_elems, torch.bfloat16, "cuda")
+    for r in range(world):
+        torch.manual_seed(r)
+        group.tensor(r).normal_()
+    tensor = group.tensor(min(3, world - 1))
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    start, stop = ctypes.c_void_p(), ctypes.c_void_p()
+    lib.tccl_event_create(ctypes.byref(start))
+    lib.tccl_event_create(ctypes.byref(stop))
+
+    fns = {
+        "all_reduce": (tccl_amd.one_shot_all_reduce, lambda n: (world + 1) * n * 2),
+        "two_shot": (tccl_amd.two_shot_all_reduce, lambda n: (world + 3) * n * 2),
+        "reduce_scatter": (tccl_amd.reduce_scatter, lambda n: (world + 1) * (n // world) * 2),
+        "all_gather": (lambda t: tccl_amd.all_gather(t, world), lambda n: 2 * world * n * 2),
+        "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel()), None),
+    }
+    fn, algo_bytes = fns[args.op]
+    size = args.max_elems
+    while size >= 2048:
+        view = tensor[:size]
+        fn(view)                                    # warm-up (the reference has none)
+        lib.tccl_event_record(start, stream)
+        for _ in range(REPS):
+            fn(view)
+        lib.tccl_event_record(stop, stream)
+        lib.tccl_event_synchronize(stop)
+        ms = ctypes.c_float()
+        lib.tccl_event_elapsed_ms(start, stop, ctypes.byref(ms))
+        per_call_ms = ms.value / REPS
+        line = f"tccl_amd {size * 2} {size * 2 / per_call_ms / 1e6:.3f} GB/s"
+        if algo_bytes is not None:
+            line += f"  (HBM {algo_bytes(size) / per_call_ms / 1e6:.1f} GB/s, {per_call_ms * 1e3:.1f} us)"
+        else:
+            line += f"  ({per_call_ms * 1e3:.1f} us)"
+        print(line, flush=True)
+        size //= 2
+    tccl_amd.unregister(group)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

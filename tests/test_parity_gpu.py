@@ -311,6 +311,21 @@ def test_all_gather_launch_shapes(unroll, flags, _gpu_hygiene):
         assert_bit_equal(tccl_amd.all_gather(g.tensor(0), 4, cfg=cfg), torch.stack(bufs), f"{block}/{unroll}")
 
 
+@pytest.mark.parametrize("world", [2, 4, 8])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+def test_two_shot_all_reduce_equals_one_shot(world, maker, _gpu_hygiene, c_oracle):
+    numel = 8 * world * 20_011
+    bufs = maker(world, numel)
+    g = upload(_gpu_hygiene, bufs)
+    want = oracle_sum(c_oracle, bufs)
+    for r in (0, world - 1):
+        assert_bit_equal(tccl_amd.two_shot_all_reduce(g.tensor(r)), want, f"two-shot rank {r}")
+        assert_bit_equal(tccl_amd.all_reduce(g.tensor(r), "two_shot"), want, "by name")
+    assert_bit_equal(tccl_amd.all_reduce(g.tensor(0)), want, "auto")
+    with pytest.raises(ValueError):
+        tccl_amd.all_reduce(g.tensor(0), "ring")
+
+
 # ------------------------------------------------------------------ double-tree node steps
 
 @pytest.mark.parametrize("children", [(False, False), (True, False), (False, True), (True, True)])
