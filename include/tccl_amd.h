@@ -57,7 +57,7 @@ typedef enum {
 typedef struct {
     int block;      /* threads per workgroup: 64, 128, 256 or 512 */
     int unroll;     /* independent 16-byte vectors per thread per iteration: 1, 2 or 4 */
-    int grid;       /* workgroups (per source row for the gather) */
+    int grid;       /* workgroups */
     int tile_iters; /* consecutive iterations a workgroup spends on one contiguous tile */
     int flags;      /* TCCL_CFG_* */
 } tccl_launch_cfg;

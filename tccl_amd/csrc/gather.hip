@@ -9,18 +9,15 @@ struct RowTable {
     const char *p[TCCL_MAX_WORLD];
 };
 
-// blockIdx.y selects the source row; the workgroups of a row tile its vectors.  Row i is
-// written at out + i * row_bytes (the [world, numel] layout of triton_all_gather.py:82).
-// The reference runs the rank loop innermost (triton_all_gather.py:54-62), so one
-// workgroup feeds `world` far-apart store streams at once; here a workgroup stays on one
-// row, which keeps each wave's loads and stores on one dense address range.
+// Row i is written at out + i * row_bytes (the [world, numel] layout of
+// triton_all_gather.py:82).  The reference runs the rank loop innermost
+// (triton_all_gather.py:54-62), so one workgroup feeds `world` far-apart store streams at
+// once; here the grid walks the rows one after the other.
 template <int UNROLL, bool NTL, bool NTS>
 __global__ void __launch_bounds__(kMaxBlock)
-pack_kernel(RowTable rows, char *out, size_t row_vecs, int tile_iters, int xcd_contiguous)
+pack_kernel(RowTable rows, int world, char *out, size_t row_vecs, int tile_iters, int xcd_contiguous)
 {
-    const int row = blockIdx.y;
-    char *const dst[1] = {out + static_cast<size_t>(row) * row_vecs * kVecBytes};
-    copy_range<1, UNROLL, NTL, NTS>(rows.p[row], dst, row_vecs, tile_iters, xcd_contiguous != 0);
+    pack_rows<UNROLL, NTL, NTS>(rows.p, world, out, row_vecs, tile_iters, xcd_contiguous != 0);
 }
 
 template <int NDST, int UNROLL, bool NTL, bool NTS>
@@ -40,7 +37,7 @@ template <int UNROLL, bool NTL, bool NTS>
 static hipError_t launch_pack(const RowTable &rows, int world, char *out, size_t row_vecs, const Shape &sh,
                               hipStream_t stream)
 {
-    hipLaunchKernelGGL((pack_kernel<UNROLL, NTL, NTS>), dim3(sh.grid, world), dim3(sh.block), 0, stream, rows, out,
+    hipLaunchKernelGGL((pack_kernel<UNROLL, NTL, NTS>), dim3(sh.grid), dim3(sh.block), 0, stream, rows, world, out,
                        row_vecs, sh.tile_iters, sh.xcd_contiguous ? 1 : 0);
     return hipGetLastError();
 }

@@ -35,9 +35,9 @@ struct Shape {
 // Fill in whatever the caller left at 0.
 //   nvec      -- 16-byte vectors of output the launch produces (per row for the gather)
 //   nsrc      -- source streams read per output vector
-//   rows      -- independent rows sharing the grid's y dimension (gather), else 1
-//   is_copy   -- a pure copy: large ones default to streaming (nt) stores, which on this
-//                memory system is worth 20 % once the output no longer fits the caches
+//   rows      -- rows of nvec vectors each that share the grid (gather), else 1
+//   is_copy   -- a pure copy: large ones get their own defaults (one workgroup per compute
+//                unit, streaming loads and stores), worth 15-20 % on this memory system
 Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows, bool is_copy = false);
 
 } // namespace tccl

@@ -387,4 +387,42 @@ __device__ __forceinline__ void copy_range(const char *src, char *const (&dst)[N
     }
 }
 
+// Pack copy: `rows` sources of row_vecs vectors each into one output, row after row.  The
+// tile index runs over all rows in row-major order, so at any moment the whole grid works
+// on one dense window of one source and one dense window of the output (two DRAM streams,
+// not 2 x rows).
+template <int UNROLL, bool NTL, bool NTS>
+__device__ __forceinline__ void pack_rows(const char *const *rows_base, int rows, char *out, size_t row_vecs,
+                                          int tile_iters, bool xcd_contiguous)
+{
+    const size_t span = static_cast<size_t>(blockDim.x) * UNROLL;
+    const size_t tile = span * static_cast<size_t>(tile_iters);
+    const size_t tiles_per_row = (row_vecs + tile - 1) / tile;
+    const size_t ntiles = tiles_per_row * static_cast<size_t>(rows);
+    for (TileWalk w(xcd_contiguous, ntiles); w.valid(); w.next()) {
+        const size_t row = w.tile() / tiles_per_row;
+        const size_t t0 = (w.tile() - row * tiles_per_row) * tile;
+        const size_t t1 = (t0 + tile < row_vecs) ? t0 + tile : row_vecs;
+        const char *src = rows_base[row];
+        char *dst = out + row * row_vecs * kVecBytes;
+        for (size_t base = t0; base < t1; base += span) {
+            if (base + span <= t1) {
+                u32x4 v[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+                    v[u] = load_vec<NTL>(src, base + static_cast<size_t>(u) * blockDim.x + threadIdx.x);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+                    store_vec<NTS>(dst, base + static_cast<size_t>(u) * blockDim.x + threadIdx.x, v[u]);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const size_t i = base + static_cast<size_t>(u) * blockDim.x + threadIdx.x;
+                    if (i < t1) store_vec<NTS>(dst, i, load_vec<NTL>(src, i));
+                }
+            }
+        }
+    }
+}
+
 } // namespace tccl
