@@ -35,6 +35,9 @@ extern "C" {
 #define TCCL_MAX_WORLD 8
 /* Largest number of node steps one tccl_tree_level() launch can take. */
 #define TCCL_MAX_JOBS 8
+/* Largest world tccl_double_tree_all_reduce() runs (a node step reads at most 3 buffers, so
+ * the tree is not bound by TCCL_MAX_WORLD). */
+#define TCCL_MAX_TREE_RANKS 64
 /* Largest world the host-side tree index math accepts. */
 #define TCCL_MAX_TREE_WORLD (1 << 20)
 
@@ -153,7 +156,7 @@ size_t tccl_double_tree_split(size_t numel, size_t esize);
  * down-sweep -- each rank copies its parent's buffer into its own buffer and its output.
  * bufs[r] is overwritten with the result (as in the reference's design, :293-294 and
  * :321-323); outs[r] (nullable entries) receive rank r's output (:324-325).  `world` is a
- * power of two, 2..TCCL_MAX_WORLD.  chunk_elems = elements per pipelining chunk
+ * power of two, 2..TCCL_MAX_TREE_RANKS.  chunk_elems = elements per pipelining chunk
  * (0 = 128 KiB worth). */
 int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs, int world, size_t numel,
                                 int dtype, size_t chunk_elems, void *stream);

@@ -224,7 +224,7 @@ extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs,
     const int esize = dtype_size(dtype);
     if (esize == 0 || bufs == nullptr) return TCCL_EINVAL;
     if (!pow2_world(world)) return TCCL_EPOW2;
-    if (world > TCCL_MAX_WORLD) return TCCL_EINVAL;
+    if (world > TCCL_MAX_TREE_RANKS) return TCCL_EINVAL;
     for (int r = 0; r < world; ++r) {
         if (bufs[r] == nullptr) return TCCL_EINVAL;
         if (!aligned16(bufs[r]) || (outs && !aligned16(outs[r]))) return TCCL_EALIGN;
@@ -242,8 +242,8 @@ extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs,
     while ((1 << height) < world) ++height;
 
     // node_height[tree][rank]: 0 = leaf, 1..height-1 = interior, height = the extra node.
-    int nbr[2][TCCL_MAX_WORLD][3];
-    int node_height[2][TCCL_MAX_WORLD];
+    int nbr[2][TCCL_MAX_TREE_RANKS][3];
+    int node_height[2][TCCL_MAX_TREE_RANKS];
     for (int r = 0; r < world; ++r) {
         int six[6];
         int rc = tccl_double_tree_indices(world, r, six);

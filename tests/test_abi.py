@@ -70,7 +70,7 @@ def test_argument_checks_return_codes_without_launching():
     assert lib.tccl_tree_level(None, 1, 0, 0, None) == -1
     assert lib.tccl_tree_level(None, 0, 9, 0, None) == -1
     assert lib.tccl_double_tree_all_reduce(good, None, 3, 64, 0, 0, None) == -3
-    assert lib.tccl_double_tree_all_reduce(good, None, 16, 64, 0, 0, None) == -1
+    assert lib.tccl_double_tree_all_reduce(good, None, 128, 64, 0, 0, None) == -1
     assert lib.tccl_double_tree_all_reduce(good, None, 2, 60, 0, 0, None) == -2
     assert lib.tccl_double_tree_all_reduce(good, None, 2, 0, 0, 0, None) == 0
     assert lib.tccl_event_create(None) == -1

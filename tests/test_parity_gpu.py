@@ -394,8 +394,7 @@ def test_tree_level_batch(_gpu_hygiene, c_oracle):
     fill(jobs[0], [x[0].data_ptr(), x[1].data_ptr(), x[2].data_ptr()], [outs[0].data_ptr(), None], n1, 0)
     fill(jobs[1], [x[3].data_ptr(), None, x[4].data_ptr()], [x[4].data_ptr(), outs[1].data_ptr()], n2, 0)   # in place + 2nd dst
     fill(jobs[2], [x[5].data_ptr(), None, None], [outs[2].data_ptr(), outs[3].data_ptr()], n1, 1)
-    fill(jobs[3], [None, None, x[5].data_ptr()], [x[5].data_ptr(), None], n2, 0)           # leaf step in place, after job 2 reads? no: same launch
-    # job 3 would race with job 2 on x[5]; give it its own buffer instead
+    # a leaf step in place on a buffer of its own (jobs of one launch must not share outputs)
     y = seeded_randn(1, n2, seed_base=99)[0]
     d_y = y.to(DEV)
     fill(jobs[3], [None, None, d_y.data_ptr()], [d_y.data_ptr(), None], n2, 0)
@@ -417,7 +416,7 @@ def test_tree_level_batch(_gpu_hygiene, c_oracle):
 
 # ------------------------------------------------------------------ full double tree
 
-@pytest.mark.parametrize("world", [2, 4, 8])
+@pytest.mark.parametrize("world", [2, 4, 8, 16, 32])
 @pytest.mark.parametrize("numel", [8, 16, 8 * 12_345, 65_536 * 4 + 8])
 def test_double_tree_all_ranks(world, numel, _gpu_hygiene, c_oracle):
     bufs = seeded_randn(world, numel, seed_base=100)
