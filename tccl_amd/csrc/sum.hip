@@ -104,6 +104,12 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
     size_t kcount;
     if (cfg && cfg->tile_iters > 0) {
         kcount = static_cast<size_t>(cfg->tile_iters) > kmax ? kmax : cfg->tile_iters;
+    } else if (NSRC <= 3 && !(cfg && cfg->grid > 0) && nvec > wgs * span * kmax) {
+        // With three sources or fewer a quarter or more of the traffic is writes and there
+        // is little left to separate: beyond one resident wave of tiles, one launch over
+        // quarter-size tiles beats a launch per wave (measured 4-13 % at 256 MiB).
+        kcount = kmax / 4;
+        wgs = (nvec + kcount * span - 1) / (kcount * span);
     } else {
         // Fewest launches that fit, then the smallest tile that covers a launch's share
         // with `wgs` workgroups, so that every launch is one full, even wave of workgroups.
@@ -114,6 +120,7 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
         if (kcount < 1) kcount = 1;
         if (kcount > kmax) kcount = kmax;
     }
+    if (wgs > (static_cast<size_t>(1) << 30)) wgs = static_cast<size_t>(1) << 30; // grid dimension limit
     const size_t tile_vec = kcount * span;
     const size_t slice_vec = wgs * tile_vec;
     const size_t tail_first = nvec * per_vec;
