@@ -157,7 +157,7 @@ size_t tccl_double_tree_split(size_t numel, size_t esize);
  * bufs[r] is overwritten with the result (as in the reference's design, :293-294 and
  * :321-323); outs[r] (nullable entries) receive rank r's output (:324-325).  `world` is a
  * power of two, 2..TCCL_MAX_TREE_RANKS.  chunk_elems = elements per pipelining chunk
- * (0 = 128 KiB worth). */
+ * (0 = 128 KiB worth); a chunk is worked on in tiles of at most 32 KiB, one workgroup each. */
 int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs, int world, size_t numel,
                                 int dtype, size_t chunk_elems, void *stream);
 

@@ -12,12 +12,14 @@ struct JobTable {
 };
 
 // One node step over its element range.  blockIdx.y selects the job; workgroup x of a job
-// takes tile x, x + gridDim.x, ...  A tile is one pipelining chunk (or a 128 KiB piece of
-// it when chunks are larger): its sources are read and reduced into registers, then the
-// result is written, the way one message of the tree pipeline would be received, reduced
-// and forwarded.
+// takes tile x, x + gridDim.x, ...  A tile is a 32 KiB piece of a pipelining chunk (the
+// whole chunk when chunks are smaller): its sources are read and reduced into registers,
+// then the result is written, the way one message of the tree pipeline would be received,
+// reduced and forwarded.  32 KiB is the measured optimum for steps with one to three
+// sources (a 128 MiB two-child step: 77 us with 32 KiB tiles, 87 us with 128 KiB tiles);
+// the tiles of one chunk are neighbours in the grid, so a chunk still completes as a unit.
 constexpr int kLevelU = 2;
-constexpr int kLevelKMax = kPhasedVecs / kLevelU;
+constexpr int kLevelKMax = 4;
 
 template <class Sum, int NDST, bool FULL>
 __device__ __forceinline__ void run_tile(const tccl_node_job &j, char *const (&dst)[NDST], size_t off, uint32_t valid,
@@ -96,7 +98,7 @@ int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_e
     const size_t span = static_cast<size_t>(kPhasedBlock) * kLevelU; // vectors per iteration
     size_t kcount = (chunk_elems / per_vec + span - 1) / span;
     if (kcount < 1) kcount = 1;
-    if (kcount > kLevelKMax) kcount = kLevelKMax; // larger chunks are walked in 128 KiB pieces
+    if (kcount > kLevelKMax) kcount = kLevelKMax; // larger chunks are walked in 32 KiB tiles
 
     JobTable t = {};
     size_t max_tiles = 0;
