@@ -161,6 +161,18 @@ size_t tccl_double_tree_split(size_t numel, size_t esize);
 int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs, int world, size_t numel,
                                 int dtype, size_t chunk_elems, void *stream);
 
+/* The same collective recorded once into a HIP graph and replayed with one launch, for
+ * callers that repeat it on the same buffers (its 2*log2(world)+1 launches cost more than
+ * its kernels below a few MiB).  No counterpart in the reference, whose whole collective
+ * is one kernel per rank.  Creating a plan allocates host and driver memory (never device
+ * memory) and does not run anything; launching it is asynchronous on `stream`.  A plan
+ * holds the addresses it was created with: the buffers must stay allocated. */
+typedef struct tccl_plan tccl_plan;
+int tccl_double_tree_plan_create(void *const *bufs, void *const *outs, int world, size_t numel,
+                                 int dtype, size_t chunk_elems, tccl_plan **plan_out);
+int tccl_plan_launch(tccl_plan *plan, void *stream);
+int tccl_plan_destroy(tccl_plan *plan);
+
 /* HIP-event helpers so a host language without HIP bindings can time launches on the very
  * stream they run on.  No counterpart in the reference (it times with torch.cuda.Event,
  * triton_reduce_scatter.py:216-226). */

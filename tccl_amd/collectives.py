@@ -185,6 +185,47 @@ def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, 
     return _run_double_tree(group, like.numel(), dtype, like, chunk_elems)
 
 
+class DoubleTreePlan:
+    """The whole double-tree all-reduce of a group recorded into a HIP graph.
+
+    ``run()`` replays it with a single launch on torch's current stream and returns the W
+    outputs (the same tensors every time; the group's buffers are overwritten with the
+    result, as by ``double_tree_all_reduce``).  Worth it when the collective is repeated on
+    the same buffers and is small enough to be bound by its launches."""
+
+    def __init__(self, group: SymmGroup, numel: Optional[int] = None, *, chunk_elems: int = 0):
+        like = group.tensors[0].reshape(-1)
+        if numel is not None:
+            like = like[:numel]
+        dtype = _sum_dtype(like)
+        assert like.numel() % _vec_elems(like) == 0, "The number of elements must be 128-bit aligned."
+        self.group = group
+        self.outputs = [torch.empty_like(like) for _ in range(group.world_size)]
+        self._out_ptrs = _lib.ptr_array([int(o.data_ptr()) for o in self.outputs])
+        self._plan = ctypes.c_void_p()
+        lib = _lib.load()
+        rc = lib.tccl_double_tree_plan_create(group.ptr_array, self._out_ptrs, group.world_size, like.numel(), dtype,
+                                              chunk_elems, ctypes.byref(self._plan))
+        _lib.check("tccl_double_tree_plan_create", rc)
+
+    def run(self) -> List[torch.Tensor]:
+        if not self._plan:
+            raise RuntimeError("plan has been closed")
+        _lib.check("tccl_plan_launch", _lib.load().tccl_plan_launch(self._plan, _stream()))
+        return self.outputs
+
+    def close(self) -> None:
+        if self._plan:
+            _lib.load().tccl_plan_destroy(self._plan)
+            self._plan = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 # BASELINE names for the same functions
 reduce_scatter = one_shot_reduce_scatter
 all_gather = one_shot_all_gather

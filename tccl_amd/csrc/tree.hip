@@ -1,5 +1,6 @@
 // tree.hip -- the double binary tree: a batch of node steps per launch, and the schedule
 // that runs the whole collective for all virtual ranks as one launch per tree level.
+#include <new>
 #include <vector>
 
 #include "host.h"
@@ -321,4 +322,64 @@ extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs,
         if (rc != TCCL_OK) return rc;
     }
     return TCCL_OK;
+}
+
+// ------------------------------------------------------------------ recorded plans
+
+struct tccl_plan {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+extern "C" int tccl_double_tree_plan_create(void *const *bufs, void *const *outs, int world, size_t numel, int dtype,
+                                            size_t chunk_elems, tccl_plan **plan_out)
+{
+    if (plan_out == nullptr) return TCCL_EINVAL;
+    *plan_out = nullptr;
+    (void)compute_units(); // device query now, not while a stream is being captured
+    hipStream_t cap = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&cap, hipStreamNonBlocking);
+    if (e != hipSuccess) return hip_code(e);
+    e = hipStreamBeginCapture(cap, hipStreamCaptureModeRelaxed);
+    if (e != hipSuccess) {
+        hipStreamDestroy(cap);
+        return hip_code(e);
+    }
+    const int rc = tccl_double_tree_all_reduce(bufs, outs, world, numel, dtype, chunk_elems, cap);
+    hipGraph_t graph = nullptr;
+    e = hipStreamEndCapture(cap, &graph); // always end the capture, also after an argument error
+    hipStreamDestroy(cap);
+    if (rc != TCCL_OK || e != hipSuccess || graph == nullptr) {
+        if (graph) hipGraphDestroy(graph);
+        return rc != TCCL_OK ? rc : (e != hipSuccess ? hip_code(e) : TCCL_EINVAL);
+    }
+    tccl_plan *plan = new (std::nothrow) tccl_plan;
+    if (plan == nullptr) {
+        hipGraphDestroy(graph);
+        return hip_code(hipErrorOutOfMemory);
+    }
+    plan->graph = graph;
+    e = hipGraphInstantiate(&plan->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        hipGraphDestroy(graph);
+        delete plan;
+        return hip_code(e);
+    }
+    *plan_out = plan;
+    return TCCL_OK;
+}
+
+extern "C" int tccl_plan_launch(tccl_plan *plan, void *stream)
+{
+    if (plan == nullptr || plan->exec == nullptr) return TCCL_EINVAL;
+    return hip_code(hipGraphLaunch(plan->exec, static_cast<hipStream_t>(stream)));
+}
+
+extern "C" int tccl_plan_destroy(tccl_plan *plan)
+{
+    if (plan == nullptr) return TCCL_EINVAL;
+    hipError_t e1 = plan->exec ? hipGraphExecDestroy(plan->exec) : hipSuccess;
+    hipError_t e2 = plan->graph ? hipGraphDestroy(plan->graph) : hipSuccess;
+    delete plan;
+    return hip_code(e1 != hipSuccess ? e1 : e2);
 }

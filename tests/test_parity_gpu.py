@@ -227,6 +227,35 @@ def test_all_reduce_256mib_per_buffer(_gpu_hygiene, c_oracle):
     assert_bit_equal(out, want, "256 MiB")
 
 
+def test_launches_follow_the_current_stream(_gpu_hygiene, c_oracle):
+    """Kernels go to torch's current stream: producer work queued on a side stream is seen
+    by the collective launched after it on that stream, with no device synchronisation in
+    between, and the default stream learns of the result through an event."""
+    world, numel = 8, 8 * 8 * 37_501
+    bufs = seeded_randn(world, numel, seed_base=77)
+    want = oracle_sum(c_oracle, bufs)
+    g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    staged = [b.to(DEV) for b in bufs]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for r in range(world):
+            g.tensor(r).zero_()
+            g.tensor(r).copy_(staged[r], non_blocking=True)     # producer, on the side stream
+        out = tccl_amd.one_shot_all_reduce(g.tensor(0))          # consumer, same stream
+        share = tccl_amd.reduce_scatter(g.tensor(1))
+        done = torch.cuda.Event()
+        done.record(side)
+    torch.cuda.current_stream().wait_event(done)
+    doubled = out.float() * 2                                    # default-stream consumer
+    torch.cuda.synchronize()
+    assert_bit_equal(out, want, "side stream")
+    per = numel // world
+    assert_bit_equal(share, want[per:2 * per], "side stream reduce-scatter")
+    assert torch.equal(doubled.cpu(), want.float() * 2)
+
+
 # ------------------------------------------------------------------ reduce-scatter
 
 @pytest.mark.parametrize("world", [2, 4, 8])
@@ -438,6 +467,34 @@ def test_double_tree_fill_rank_and_second_collective(_gpu_hygiene):
     # every buffer now holds 28; the next collective sums those: 8 * 28
     for r in range(world):
         assert tccl_amd.double_tree_all_reduce(g.tensor(r)).eq(224).all().item()
+
+
+@pytest.mark.parametrize("world,numel", [(8, 8 * 4099), (4, 65_536 * 3), (16, 8 * 513)])
+def test_double_tree_plan_replays(world, numel, _gpu_hygiene, c_oracle):
+    """The recorded plan against the eager schedule and the oracle, replayed several times
+    with other work and synchronisations in between; every replay is checked."""
+    g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    plan = tccl_amd.DoubleTreePlan(g)
+    for rep in range(4):
+        bufs = seeded_randn(world, numel, seed_base=1000 + 10 * rep)
+        _, outs = c_oracle.double_tree_all_reduce_bf16([np_bits(b) for b in bufs])
+        want = from_np_bits(outs[0])
+        for r in range(world):
+            g.tensor(r).copy_(bufs[r])
+        got = plan.run()
+        torch.cuda.synchronize()
+        for r in range(world):
+            assert_bit_equal(got[r], want, f"replay {rep} output {r}")
+            assert_bit_equal(g.tensor(r), want, f"replay {rep} buffer {r}")
+        # eager work between replays: the same collective without the plan
+        for r in range(world):
+            g.tensor(r).copy_(bufs[r])
+        eager = tccl_amd.double_tree_all_reduce_world(g)
+        assert_bit_equal(eager[0], want, f"eager after replay {rep}")
+    plan.close()
+    with pytest.raises(RuntimeError):
+        plan.run()
 
 
 def test_double_tree_f32_and_chunk_sizes(_gpu_hygiene, c_oracle):
