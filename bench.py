@@ -44,6 +44,8 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     p.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU work budget for the baseline leg")
+    p.add_argument("--no-other-ops", action="store_true",
+                   help="skip the short timings of reduce-scatter, all-gather and the tree node steps")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run 20 plain copies of 256 MiB (tccl_tree_copy_step), so that a rocprofv3 --pmc "
                         "run of this command holds a kernel of known traffic to scale the counters by")
@@ -245,6 +247,9 @@ def main():
         }
         del bufs_cpu
 
+    if not args.no_other_ops:
+        result["other_ops"] = other_ops(torch, tccl_amd, lib, device)
+
     if args.calibrate_copy:
         nbytes = 256 << 20
         src = torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device=device)
@@ -260,6 +265,75 @@ def main():
         run_sweep(torch, tccl_amd, lib, device)
 
     print(json.dumps(result), flush=True)
+
+
+def other_ops(torch, tccl_amd, lib, device):
+    """The other operations of the path at their BASELINE shapes, bf16: GB/s on algorithmic
+    bytes from HIP events (30 launches after 5 warm-ups).  Each rotates over enough disjoint
+    buffers that nothing is served from the 256 MB memory-side cache."""
+    import gc
+    from tccl_amd import _lib
+    out = {}
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    # reduce-scatter: W=8 inputs of 67,108,864 elements, every rank's share in turn (8 x 144 MiB touched)
+    g = make_world(tccl_amd, torch, 8, 67_108_864, torch.bfloat16, device)
+    turn = [0]
+
+    def rs():
+        turn[0] += 1
+        return tccl_amd.reduce_scatter(g.tensor(turn[0] % 8))
+    _, ms = time_steps(torch, lib, rs, 32, 8)
+    out["reduce_scatter_w8_64Mi_el_gbs"] = round(9 * (67_108_864 // 8) * 2 / (ms * 1e-3) / 1e9, 1)
+    tccl_amd.unregister(g)
+    del g
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    # all-gather: W=8 x 8,388,608 elements, two groups alternating (2 x 256 MiB touched)
+    gs = [make_world(tccl_amd, torch, 8, 8_388_608, torch.bfloat16, device) for _ in range(2)]
+
+    def ag():
+        turn[0] += 1
+        return tccl_amd.all_gather(gs[turn[0] % 2].tensor(0), 8)
+    _, ms = time_steps(torch, lib, ag, 30, 6)
+    out["all_gather_w8_8Mi_el_gbs"] = round(2 * 8 * 8_388_608 * 2 / (ms * 1e-3) / 1e9, 1)
+    for g in gs:
+        tccl_amd.unregister(g)
+    del gs
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    # tree node steps on 128 MiB halves in 128 KiB chunks: four different jobs in turn (2 GiB touched)
+    half = 67_108_864
+    bufs = [torch.randn(half, dtype=torch.float32, device=device).to(torch.bfloat16) for _ in range(12)]
+    jobs = [(_lib.NodeJob * 1)() for _ in range(4)]
+
+    def set_reduce():
+        for i, j in enumerate(jobs):
+            j[0].src[0], j[0].src[1], j[0].src[2] = bufs[3 * i + 1].data_ptr(), bufs[3 * i + 2].data_ptr(), bufs[3 * i].data_ptr()
+            j[0].dst[0], j[0].dst[1] = bufs[3 * i].data_ptr(), None
+            j[0].numel, j[0].is_copy = half, 0
+
+    def set_copy():
+        for i, j in enumerate(jobs):
+            j[0].src[0], j[0].src[1], j[0].src[2] = bufs[3 * i].data_ptr(), None, None
+            j[0].dst[0], j[0].dst[1] = bufs[3 * i + 1].data_ptr(), bufs[3 * i + 2].data_ptr()
+            j[0].numel, j[0].is_copy = half, 1
+
+    def level():
+        turn[0] += 1
+        return lib.tccl_tree_level(jobs[turn[0] % 4], 1, 0, 65_536, stream)
+    set_reduce()
+    _, ms = time_steps(torch, lib, level, 32, 8)
+    out["tree_reduce_step_2_children_128MiB_gbs"] = round(4 * half * 2 / (ms * 1e-3) / 1e9, 1)
+    set_copy()
+    _, ms = time_steps(torch, lib, level, 32, 8)
+    out["tree_copy_step_2_destinations_128MiB_gbs"] = round(3 * half * 2 / (ms * 1e-3) / 1e9, 1)
+    del bufs
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
 
 
 def run_sweep(torch, tccl_amd, lib, device):

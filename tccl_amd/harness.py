@@ -21,7 +21,8 @@ REPS = 10          # as in the reference
 
 def main(argv=None) -> int:
     p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    p.add_argument("op", choices=["all_reduce", "reduce_scatter", "all_gather", "double_tree", "two_shot"])
+    p.add_argument("op", choices=["all_reduce", "reduce_scatter", "all_gather", "double_tree", "double_tree_plan",
+                                  "two_shot"])
     p.add_argument("--world", type=int, default=8)
     p.add_argument("--max-elems", type=int, default=256 * 1024 * 1024 // 2,
                    help="largest element count per rank (bf16); halved down to 2,048")
@@ -48,10 +49,14 @@ def main(argv=None) -> int:
         "all_gather": (lambda t: tccl_amd.all_gather(t, world), lambda n: 2 * world * n * 2),
         "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel()), None),
     }
-    fn, algo_bytes = fns[args.op]
     size = args.max_elems
     while size >= 2048:
         view = tensor[:size]
+        if args.op == "double_tree_plan":       # one recorded plan per size, replayed
+            plan = tccl_amd.DoubleTreePlan(group, size)
+            fn, algo_bytes = (lambda t: plan.run()), None
+        else:
+            fn, algo_bytes = fns[args.op]
         fn(view)                                    # warm-up (the reference has none)
         lib.tccl_event_record(start, stream)
         for _ in range(REPS):

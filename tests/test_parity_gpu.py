@@ -319,6 +319,16 @@ def test_all_gather_equals_stack(maker, numel, _gpu_hygiene):
     assert_bit_equal(out, torch.stack(bufs), maker.__name__)
 
 
+def test_all_gather_fill_rank(_gpu_hygiene):
+    """The reference's (commented) all-gather test, triton_all_gather.py:117-133: every rank
+    fills 2,048 elements with its rank; the result is the stack of those."""
+    world = 8
+    g = upload(_gpu_hygiene, [torch.full((2048,), float(r), dtype=torch.bfloat16) for r in range(world)])
+    want = torch.stack([torch.full((2048,), float(r), dtype=torch.bfloat16) for r in range(world)])
+    for r in range(world):
+        assert_bit_equal(tccl_amd.one_shot_all_gather(g.tensor(r), world), want, f"rank {r}")
+
+
 @pytest.mark.parametrize("world", [1, 2, 3, 5, 8])
 def test_all_gather_worlds_shapes_and_nan_payloads(world, _gpu_hygiene):
     rng = np.random.default_rng(world)
