@@ -89,6 +89,58 @@ __global__ void __launch_bounds__(kPhasedBlock) tree_level_kernel(JobTable jobs,
         run_job<Sum, 1, FULL>(j, kcount);
 }
 
+// A level made of copy steps only (every level of the down-sweep): the jobs are walked one
+// after the other by a small persistent grid, 16 KiB per workgroup per step, loads and
+// stores streaming.  The whole GPU then works on one source window and its destination
+// windows at a time; for copies that beats read-then-write tiles by 5-6 % and running the
+// jobs side by side by more.
+constexpr int kCopyU = 4;
+
+__global__ void __launch_bounds__(kPhasedBlock) tree_copy_level_kernel(JobTable jobs, int njobs, int esize)
+{
+    constexpr size_t span_bytes = static_cast<size_t>(kPhasedBlock) * kCopyU * kVecBytes;
+    size_t spans[TCCL_MAX_JOBS];
+    size_t total = 0;
+#pragma unroll
+    for (int i = 0; i < TCCL_MAX_JOBS; ++i) {
+        spans[i] = i < njobs ? (jobs.job[i].numel * esize + span_bytes - 1) / span_bytes : 0;
+        total += spans[i];
+    }
+    const uint32_t lane_off = threadIdx.x * kVecBytes;
+    for (size_t g = blockIdx.x; g < total; g += gridDim.x) {
+        int ji = 0;
+        size_t local = g;
+#pragma unroll
+        for (int i = 0; i < TCCL_MAX_JOBS - 1; ++i) {
+            if (ji == i && local >= spans[i]) {
+                local -= spans[i];
+                ji = i + 1;
+            }
+        }
+        const tccl_node_job &j = jobs.job[ji];
+        const size_t bytes = j.numel * esize;
+        const size_t off = local * span_bytes;
+        const size_t left = bytes - off;
+        const uint32_t valid = static_cast<uint32_t>(left < span_bytes ? left : span_bytes);
+        const __amdgpu_buffer_rsrc_t rs = tile_rsrc(static_cast<const char *>(j.src[0]) + off, valid);
+        u32x4 v[kCopyU];
+#pragma unroll
+        for (int u = 0; u < kCopyU; ++u)
+            v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxLoadStream);
+        const __amdgpu_buffer_rsrc_t r0 = tile_rsrc(static_cast<char *>(j.dst[0]) + off, valid);
+#pragma unroll
+        for (int u = 0; u < kCopyU; ++u)
+            __builtin_amdgcn_raw_buffer_store_b128(v[u], r0, u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxLoadStream);
+        if (j.dst[1] != nullptr) {
+            const __amdgpu_buffer_rsrc_t r1 = tile_rsrc(static_cast<char *>(j.dst[1]) + off, valid);
+#pragma unroll
+            for (int u = 0; u < kCopyU; ++u)
+                __builtin_amdgcn_raw_buffer_store_b128(v[u], r1, u * (kPhasedBlock * kVecBytes) + lane_off, 0,
+                                                       kAuxLoadStream);
+        }
+    }
+}
+
 int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_elems, hipStream_t stream)
 {
     const int esize = dtype_size(dtype);
@@ -103,6 +155,8 @@ int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_e
 
     JobTable t = {};
     size_t max_tiles = 0;
+    bool all_copies = true;
+    size_t copy_spans = 0;
     for (int i = 0; i < njobs; ++i) {
         const tccl_node_job &j = jobs[i];
         if (j.dst[0] == nullptr) return TCCL_EINVAL;
@@ -112,9 +166,19 @@ int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_e
         if (!aligned16(j.dst[0]) || !aligned16(j.dst[1])) return TCCL_EALIGN;
         if (j.is_copy && (j.numel % per_vec) != 0) return TCCL_EALIGN;
         t.job[i] = j;
+        all_copies = all_copies && j.is_copy;
+        copy_spans += (j.numel * esize + kPhasedBlock * kCopyU * kVecBytes - 1) / (kPhasedBlock * kCopyU * kVecBytes);
         const size_t nvec = j.numel / per_vec;
         const size_t tiles = (nvec + span * kcount - 1) / (span * kcount);
         if (tiles > max_tiles) max_tiles = tiles;
+    }
+    if (all_copies) {
+        if (copy_spans == 0) return TCCL_OK;
+        size_t wgs = static_cast<size_t>(compute_units());
+        if (wgs > copy_spans) wgs = copy_spans;
+        hipLaunchKernelGGL(tree_copy_level_kernel, dim3(static_cast<unsigned>(wgs)), dim3(kPhasedBlock), 0, stream, t,
+                           njobs, esize);
+        return hip_code(hipGetLastError());
     }
     if (max_tiles == 0) max_tiles = 1; // ragged tails only
     if (max_tiles > 0x7FFFFFFFu) max_tiles = 0x7FFFFFFFu;
