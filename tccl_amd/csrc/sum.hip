@@ -104,11 +104,13 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
     size_t kcount;
     if (cfg && cfg->tile_iters > 0) {
         kcount = static_cast<size_t>(cfg->tile_iters) > kmax ? kmax : cfg->tile_iters;
-    } else if (NSRC <= 3 && !(cfg && cfg->grid > 0) && nvec > wgs * span * kmax) {
+    } else if (NSRC <= 3 && !(cfg && cfg->grid > 0) &&
+               nvec * kVecBytes >= (static_cast<size_t>(NSRC <= 2 ? 48 : 96) << 20)) {
         // With three sources or fewer a quarter or more of the traffic is writes and there
-        // is little left to separate: beyond one resident wave of tiles, one launch over
-        // quarter-size tiles beats a launch per wave (measured 4-13 % at 256 MiB).
-        kcount = kmax / 4;
+        // is little left to separate: on large inputs one launch over 16 KiB tiles beats a
+        // launch per resident wave of big tiles (measured on buffers rotated so that
+        // nothing is cached: +3 % with three sources, +6-8 % with one or two).
+        kcount = kmax / 8 > 0 ? kmax / 8 : 1;
         wgs = (nvec + kcount * span - 1) / (kcount * span);
     } else {
         // Fewest launches that fit, then the smallest tile that covers a launch's share
