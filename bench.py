@@ -268,7 +268,7 @@ def main():
 
 
 def other_ops(torch, tccl_amd, lib, device):
-    """The other operations of the path at their BASELINE shapes, bf16: GB/s on algorithmic
+    """The other operations of the path at their full benchmark shapes, bf16: GB/s on algorithmic
     bytes from HIP events (30 launches after 5 warm-ups).  Each rotates over enough disjoint
     buffers that nothing is served from the 256 MB memory-side cache."""
     import gc
@@ -337,7 +337,7 @@ def other_ops(torch, tccl_amd, lib, device):
 
 
 def run_sweep(torch, tccl_amd, lib, device):
-    """Every op at its BASELINE configuration and the all-reduce size sweep; JSON lines on
+    """Every op at its full benchmark shape and the all-reduce size sweep; JSON lines on
     stderr (GB/s on algorithmic bytes from HIP events; p50 us per launch)."""
     import gc
 

@@ -226,6 +226,6 @@ class DoubleTreePlan:
             pass
 
 
-# BASELINE names for the same functions
+# short names for the same functions
 reduce_scatter = one_shot_reduce_scatter
 all_gather = one_shot_all_gather

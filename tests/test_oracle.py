@@ -163,7 +163,7 @@ def test_f32_oracles_agree(world, c_oracle):
 
 
 def test_torch_ref_matches_c_at_config1_size(c_oracle):
-    """BASELINE config 1 shape: W=8 buffers of 4,194,304 bf16 ~N(0,1), seed = rank."""
+    """Benchmark shape 1: W=8 buffers of 4,194,304 bf16 ~N(0,1), seed = rank."""
     bufs = seeded_randn(8, 4_194_304)
     t = torch_ref.all_reduce(bufs)
     c = c_oracle.all_reduce_bf16([np_bits(b) for b in bufs])

@@ -190,7 +190,7 @@ def test_all_reduce_directed_bit_patterns(_gpu_hygiene, c_oracle):
 
 
 def test_all_reduce_config1_vs_torch_cpu_reference(_gpu_hygiene, c_oracle):
-    """BASELINE config 1: W=8 x 4,194,304 bf16 ~N(0,1), seed = rank, against the torch CPU
+    """Benchmark shape 1: W=8 x 4,194,304 bf16 ~N(0,1), seed = rank, against the torch CPU
     reference (and the C oracle)."""
     bufs = seeded_randn(8, 4_194_304)
     g = upload(_gpu_hygiene, bufs)
@@ -202,7 +202,7 @@ def test_all_reduce_config1_vs_torch_cpu_reference(_gpu_hygiene, c_oracle):
 
 @pytest.mark.parametrize("world", [2, 4, 8])
 def test_all_reduce_sweep_sizes(world, _gpu_hygiene, c_oracle):
-    """BASELINE config 2 sweep: 16 KiB .. 64 MiB per buffer in powers of 4, using prefix
+    """Benchmark sweep (shape 2): 16 KiB .. 64 MiB per buffer in powers of 4, using prefix
     views of one allocation (as the reference's benchmarks slice tensor[:size])."""
     top = (64 << 20) // 2
     bufs = seeded_randn(world, top)
@@ -281,7 +281,7 @@ def test_reduce_scatter_every_rank(world, maker, _gpu_hygiene, c_oracle):
 
 
 def test_reduce_scatter_config3(_gpu_hygiene, c_oracle):
-    """BASELINE config 3: W=8 inputs of 67,108,864 bf16 ~N(0,1), rank 3's 8,388,608-element
+    """Benchmark shape 3: W=8 inputs of 67,108,864 bf16 ~N(0,1), rank 3's 8,388,608-element
     share; then the same shapes in fp32 ~U(-1,1)."""
     world, numel, rank = 8, 67_108_864, 3
     per = numel // world
@@ -309,7 +309,7 @@ def test_reduce_scatter_fill_rank(_gpu_hygiene):
 @pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform, seeded_int8], ids=["bf16", "f32", "int8"])
 @pytest.mark.parametrize("numel", [16, 4096, 8_388_608])
 def test_all_gather_equals_stack(maker, numel, _gpu_hygiene):
-    """BASELINE config 4 (numel = 8,388,608) and smaller; expected value as in
+    """Benchmark shape 4 (numel = 8,388,608) and smaller; expected value as in
     triton_all_gather.py:128."""
     world = 8
     bufs = maker(world, numel)
@@ -519,7 +519,7 @@ def test_double_tree_f32_and_chunk_sizes(_gpu_hygiene, c_oracle):
 
 
 def test_double_tree_config5_properties(_gpu_hygiene, c_oracle):
-    """BASELINE config 5 shape: W=8 x 134,217,728 bf16 (256 MiB each), halves of
+    """Benchmark shape 5: W=8 x 134,217,728 bf16 (256 MiB each), halves of
     67,108,864 elements, 65,536-element chunks.  Checked by size-independent properties:
     all 8 outputs and all 8 buffers are bit-identical, and windows of the result equal the
     oracle run on the same windows of the inputs."""

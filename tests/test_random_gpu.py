@@ -1,0 +1,119 @@
+"""Seeded random cases on the GPU: every entry point with random worlds, sizes, dtypes and
+launch overrides against the C oracle, bit for bit.  The case list is fixed by the seed, so
+a failure names a reproducible case."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import tccl_amd
+from tccl_amd import _lib
+from helpers import assert_bit_equal, from_np_bits, np_bits
+from oracle import torch_ref
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _cases(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        world = int(rng.integers(1, 9))
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+        per_vec = 16 // (2 if dtype == torch.bfloat16 else 4)
+        scale = int(rng.choice([1, 1, 1, 40, 40, 700, 9000]))
+        nvec = int(rng.integers(0, 1 + 97 * scale))
+        ragged = int(rng.integers(0, per_vec)) if rng.random() < 0.4 else 0
+        flags = int(rng.choice([0, 0, 1, 2, 3, 4, 16, 16 | 3, 32, 32, 32]))
+        cfg = dict(block=int(rng.choice([0, 64, 128, 256, 512])), unroll=int(rng.choice([0, 1, 2, 4, 8])),
+                   grid=int(rng.choice([0, 0, 1, 3, 8, 64, 1000])), tile_iters=int(rng.choice([0, 0, 1, 2, 5, 16, 32])),
+                   flags=flags)
+        out.append((i, world, dtype, nvec * per_vec + ragged, cfg))
+    return out
+
+
+def _inputs(world, numel, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    n = max(numel, 1)
+    if dtype == torch.bfloat16:
+        return [torch.randn(n, generator=g).to(torch.bfloat16) for _ in range(world)]
+    return [torch.rand(n, generator=g) * 2 - 1 for _ in range(world)]
+
+
+def _oracle(c_oracle, bufs):
+    if bufs[0].dtype == torch.bfloat16:
+        return from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs]))
+    return torch.from_numpy(c_oracle.all_reduce_f32([b.numpy() for b in bufs]))
+
+
+@pytest.mark.parametrize("case", _cases(80, 20240607), ids=lambda c: f"case{c[0]}")
+def test_random_all_reduce_and_reduce_scatter(case, c_oracle):
+    i, world, dtype, numel, cfgd = case
+    lib = tccl_amd.load_library()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    bufs = _inputs(world, numel, dtype, 1000 + i)
+    dev = [b.to(DEV) for b in bufs]
+    ptrs = _lib.ptr_array([d.data_ptr() for d in dev])
+    dt = _lib.TCCL_BF16 if dtype == torch.bfloat16 else _lib.TCCL_F32
+    cfg = tccl_amd.LaunchCfg(**cfgd)
+    out = torch.full((numel + 32,), 3.0, dtype=dtype, device=DEV)
+    print(f"case {i}: world={world} dtype={dtype} numel={numel} cfg={cfgd}", flush=True)
+    assert lib.tccl_all_reduce_sum_ex(ptrs, world, out.data_ptr(), numel, dt, stream, ctypes.byref(cfg)) == 0
+    want = _oracle(c_oracle, [b[:numel].contiguous() for b in bufs]) if numel else bufs[0][:0]
+    assert_bit_equal(out[:numel], want, "all-reduce")
+    assert out[numel:].eq(3.0).all().item(), "wrote past the end"
+    # reduce-scatter of the same buffers for a random rank, when the share is vector-aligned
+    per_vec = 16 // bufs[0].element_size()
+    total = (numel // (per_vec * world)) * per_vec * world
+    if total:
+        rank = i % world
+        per = total // world
+        share = torch.full((per + 32,), 3.0, dtype=dtype, device=DEV)
+        assert lib.tccl_reduce_scatter_sum_ex(ptrs, world, rank, share.data_ptr(), total, dt, stream,
+                                              ctypes.byref(cfg)) == 0
+        w = _oracle(c_oracle, [b[rank * per:(rank + 1) * per].contiguous() for b in bufs])
+        assert_bit_equal(share[:per], w, "reduce-scatter")
+        assert share[per:].eq(3.0).all().item()
+
+
+@pytest.mark.parametrize("case", _cases(40, 77), ids=lambda c: f"case{c[0]}")
+def test_random_all_gather_and_tree_steps(case, c_oracle):
+    i, world, dtype, numel, cfgd = case
+    lib = tccl_amd.load_library()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    per_vec = 16 // (2 if dtype == torch.bfloat16 else 4)
+    numel = numel // per_vec * per_vec                       # copies take whole vectors only
+    bufs = _inputs(world, numel, dtype, 5000 + i)
+    dev = [b[:numel].contiguous().to(DEV) for b in bufs]
+    print(f"case {i}: world={world} dtype={dtype} numel={numel} cfg={cfgd}", flush=True)
+    if numel:
+        ptrs = _lib.ptr_array([d.data_ptr() for d in dev])
+        cfgd = dict(cfgd, unroll=cfgd["unroll"] if cfgd["unroll"] != 8 else 4, flags=cfgd["flags"] & 15)
+        cfg = tccl_amd.LaunchCfg(**cfgd)
+        out = torch.zeros((world, numel), dtype=dtype, device=DEV)
+        nbytes = numel * bufs[0].element_size()
+        assert lib.tccl_all_gather_ex(ptrs, world, out.data_ptr(), nbytes, stream, ctypes.byref(cfg)) == 0
+        assert_bit_equal(out, torch.stack([b[:numel] for b in bufs]), "all-gather")
+    if not numel:
+        return
+    # one tree reduce step with the children this case's world allows, in place
+    dt = _lib.TCCL_BF16 if dtype == torch.bfloat16 else _lib.TCCL_F32
+    own = bufs[0][:numel].contiguous()
+    c0 = bufs[1][:numel].contiguous() if world >= 2 and i % 2 == 0 else None
+    c1 = bufs[2][:numel].contiguous() if world >= 3 and i % 3 != 0 else None
+    d_own = own.to(DEV)
+    d0 = c0.to(DEV) if c0 is not None else None
+    d1 = c1.to(DEV) if c1 is not None else None
+    rc = lib.tccl_tree_reduce_step(d_own.data_ptr(), d0.data_ptr() if d0 is not None else None,
+                                   d1.data_ptr() if d1 is not None else None, d_own.data_ptr(), numel, dt, stream)
+    assert rc == 0
+    assert_bit_equal(d_own, torch_ref.tree_reduce_step(own, c0, c1), "tree reduce step in place")
+    # and the copy step into two destinations
+    a = torch.zeros_like(d_own)
+    b = torch.zeros_like(d_own)
+    assert lib.tccl_tree_copy_step(d_own.data_ptr(), a.data_ptr(), b.data_ptr(), numel * own.element_size(),
+                                   stream) == 0
+    assert_bit_equal(a, d_own, "copy dst0")
+    assert_bit_equal(b, d_own, "copy dst1")
