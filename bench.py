@@ -204,7 +204,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 in/out, fp32 accumulate",
+        "dtype": "f32",                      # the sums are accumulated in fp32 ...
+        "io_dtype": "bf16",                  # ... over bf16 inputs, rounded once to a bf16 output
         "data": "synthetic N(0,1), seeded per virtual rank, resident in HBM",
         "config": {"workload": "one-shot all-reduce sum, W=8 virtual ranks, 64 MiB bf16 per buffer "
                                "(33,554,432 elements), one MI355X",

@@ -130,13 +130,13 @@ __global__ void __launch_bounds__(kPhasedBlock) tree_copy_level_kernel(JobTable 
         const __amdgpu_buffer_rsrc_t r0 = tile_rsrc(static_cast<char *>(j.dst[0]) + off, valid);
 #pragma unroll
         for (int u = 0; u < kCopyU; ++u)
-            __builtin_amdgcn_raw_buffer_store_b128(v[u], r0, u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxLoadStream);
+            __builtin_amdgcn_raw_buffer_store_b128(v[u], r0, u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxStoreNt);
         if (j.dst[1] != nullptr) {
             const __amdgpu_buffer_rsrc_t r1 = tile_rsrc(static_cast<char *>(j.dst[1]) + off, valid);
 #pragma unroll
             for (int u = 0; u < kCopyU; ++u)
                 __builtin_amdgcn_raw_buffer_store_b128(v[u], r1, u * (kPhasedBlock * kVecBytes) + lane_off, 0,
-                                                       kAuxLoadStream);
+                                                       kAuxStoreNt);
         }
     }
 }

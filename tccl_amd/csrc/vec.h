@@ -235,7 +235,8 @@ __device__ __forceinline__ void sum_range(const char *const (&src)[NSRC], char *
 constexpr int kPhasedBlock = 256; // lanes per workgroup
 constexpr int kPhasedVecs = 32;   // result vectors a lane holds before it writes (128 VGPRs)
 constexpr int kAuxLoadStream = 2;   // cache policy of the loads: nt (stream through L2)
-constexpr int kAuxStoreStream = 16; // cache policy of the stores: sc1 (write through to memory)
+constexpr int kAuxStoreStream = 16; // cache policy of a tile's result stores: sc1 (write through to memory)
+constexpr int kAuxStoreNt = 2;      // cache policy of the stores of streaming copies: nt
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const char *tile_start, uint32_t valid_bytes)
 {

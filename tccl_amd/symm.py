@@ -94,13 +94,16 @@ def rendezvous(tensor: torch.Tensor) -> SymmHandle:
     ``tensor`` may be a rank's whole buffer or a view that starts at its first element
     (the reference's benchmarks pass ``tensor[:size]``, triton_reduce_scatter.py:222); the
     element count of a collective is taken from the tensor, the addresses from the group."""
-    base = int(tensor.untyped_storage().data_ptr())
-    hit = _registry.get(base)
+    # Fast path: a view that starts at the buffer's first element has the buffer's address.
+    hit = _registry.get(tensor.data_ptr())
     group = hit[0]() if hit is not None else None
     if group is None:
-        raise RuntimeError("tensor does not belong to a registered symmetric group "
-                           "(allocate it with tccl_amd.empty_world or register the buffers)")
-    if tensor.data_ptr() != base:
+        base = int(tensor.untyped_storage().data_ptr())
+        hit = _registry.get(base)
+        group = hit[0]() if hit is not None else None
+        if group is None:
+            raise RuntimeError("tensor does not belong to a registered symmetric group "
+                               "(allocate it with tccl_amd.empty_world or register the buffers)")
         raise RuntimeError("a collective must be given a view that starts at the buffer's first element")
     if not tensor.is_contiguous():
         raise RuntimeError("a collective must be given a contiguous view")
