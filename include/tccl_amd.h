@@ -161,6 +161,17 @@ size_t tccl_double_tree_split(size_t numel, size_t esize);
 int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs, int world, size_t numel,
                                 int dtype, size_t chunk_elems, void *stream);
 
+/* The same collective in ONE launch, for worlds of 2, 4 or 8 whose buffers all live on this
+ * GPU: each lane loads its 16-byte vector from all `world` buffers, reduces it in registers
+ * in the tree's order with the tree's rounding (one rounding per node, exactly the values
+ * the node steps produce), and stores the result into every buffer and every output.  It
+ * moves world reads + 2*world writes per element instead of the schedule's level-by-level
+ * traffic and needs no ordering between launches, which is what bounds small inputs.  No
+ * counterpart in the reference (a rank there cannot read every peer's buffer for free);
+ * it leaves memory in the same final state as tccl_double_tree_all_reduce(). */
+int tccl_double_tree_all_reduce_fused(void *const *bufs, void *const *outs, int world, size_t numel,
+                                      int dtype, void *stream);
+
 /* The same collective recorded once into a HIP graph and replayed with one launch, for
  * callers that repeat it on the same buffers (its 2*log2(world)+1 launches cost more than
  * its kernels below a few MiB).  No counterpart in the reference, whose whole collective

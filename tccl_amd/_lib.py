@@ -70,6 +70,7 @@ SIGNATURES = {
     "tccl_double_tree_indices": (_I, [_I, _I, ctypes.POINTER(_I)]),
     "tccl_double_tree_split": (_SZ, [_SZ, _SZ]),
     "tccl_double_tree_all_reduce": (_I, [_PP, _PP, _I, _SZ, _I, _SZ, _P]),
+    "tccl_double_tree_all_reduce_fused": (_I, [_PP, _PP, _I, _SZ, _I, _P]),
     "tccl_double_tree_plan_create": (_I, [_PP, _PP, _I, _SZ, _I, _SZ, _PP]),
     "tccl_plan_launch": (_I, [_P, _P]),
     "tccl_plan_destroy": (_I, [_P]),

@@ -137,18 +137,35 @@ def all_reduce(tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
     raise ValueError(f"unknown all-reduce algorithm {algorithm!r}")
 
 
+# Below this many bytes per buffer the level schedule is bound by its 2*log2(W)+1 dependent
+# launches (about 37 us for W=8 whatever the size) and the one-launch kernel is used instead.
+FUSED_TREE_MAX_BYTES = 8 << 20
+
+
 def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tensor,
-                     chunk_elems: int) -> List[torch.Tensor]:
-    outputs = [torch.empty_like(like) for _ in range(group.world_size)]
+                     chunk_elems: int, fused: Optional[bool] = None) -> List[torch.Tensor]:
+    # one allocation for all W outputs (rows are 16-byte aligned: numel is whole vectors)
+    stacked = torch.empty((group.world_size,) + tuple(like.shape), dtype=like.dtype, device=like.device)
+    outputs = list(stacked.unbind(0))
     lib = _lib.load()
-    out_ptrs = _lib.ptr_array([int(o.data_ptr()) for o in outputs])
-    rc = lib.tccl_double_tree_all_reduce(group.ptr_array, out_ptrs, group.world_size, numel, dtype, chunk_elems,
-                                         _stream())
-    _lib.check("tccl_double_tree_all_reduce", rc)
+    row_bytes = like.numel() * like.element_size()
+    first = int(stacked.data_ptr())
+    out_ptrs = _lib.ptr_array([first + r * row_bytes for r in range(group.world_size)])
+    if fused is None:
+        fused = group.world_size <= 8 and numel * like.element_size() <= FUSED_TREE_MAX_BYTES
+    if fused:
+        rc = lib.tccl_double_tree_all_reduce_fused(group.ptr_array, out_ptrs, group.world_size, numel, dtype,
+                                                   _stream())
+        _lib.check("tccl_double_tree_all_reduce_fused", rc)
+    else:
+        rc = lib.tccl_double_tree_all_reduce(group.ptr_array, out_ptrs, group.world_size, numel, dtype, chunk_elems,
+                                             _stream())
+        _lib.check("tccl_double_tree_all_reduce", rc)
     return outputs
 
 
-def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0) -> torch.Tensor:
+def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
+                           fused: Optional[bool] = None) -> torch.Tensor:
     """All-reduce over two complementary binary trees, one per half of the elements.
 
     Mirrors ``double_tree_all_reduce`` (triton_double_tree_allreduce.py:338-370) as its
@@ -160,7 +177,11 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0) -> tor
     A collective is one call per rank.  On one GPU the first rank to call runs the node
     steps of *all* virtual ranks (the ranks' buffers are overwritten with the result, as
     in the reference's design) and gets its output; the other ranks' outputs wait in the
-    group until those ranks call.  A rank calling again starts the next collective."""
+    group until those ranks call.  A rank calling again starts the next collective.
+
+    ``fused``: False = one launch per tree level (the node-step kernels), True = the whole
+    tree in one launch (worlds of 2, 4, 8; same values, same final memory), None = the
+    one-launch kernel up to ``FUSED_TREE_MAX_BYTES`` per buffer, the level schedule above."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
     symm = rendezvous(tensor)
@@ -168,13 +189,13 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0) -> tor
     pending = group.pending_outputs.pop(symm.rank, None)
     if pending is not None and pending.shape == tensor.shape:
         return pending
-    outputs = _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems)
+    outputs = _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems, fused)
     group.pending_outputs = {r: o for r, o in enumerate(outputs) if r != symm.rank}
     return outputs[symm.rank]
 
 
 def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *,
-                                 chunk_elems: int = 0) -> List[torch.Tensor]:
+                                 chunk_elems: int = 0, fused: Optional[bool] = None) -> List[torch.Tensor]:
     """One whole collective for every virtual rank of ``group``; returns the W outputs."""
     like = group.tensors[0].reshape(-1)
     if numel is not None:
@@ -182,7 +203,7 @@ def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, 
     dtype = _sum_dtype(like)
     assert like.numel() % _vec_elems(like) == 0, "The number of elements must be 128-bit aligned."
     group.pending_outputs.clear()
-    return _run_double_tree(group, like.numel(), dtype, like, chunk_elems)
+    return _run_double_tree(group, like.numel(), dtype, like, chunk_elems, fused)
 
 
 class DoubleTreePlan:

@@ -388,6 +388,124 @@ extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs,
     return TCCL_OK;
 }
 
+// ------------------------------------------------------------------ the whole tree in one launch
+namespace tccl {
+
+// Labels are ranks of tree a; tree b is tree a with every label lowered by one (mod W), so
+// the lane handling a vector of the second half simply loads label l from rank (l-1) mod W.
+
+// Result of the subtree rooted at interior-or-leaf label R (R >= 1), LOW = lowest set bit of
+// R: round(0 + node(R - LOW/2) + node(R + LOW/2) + x[R]); a leaf (LOW == 1) is
+// round(0 + x[R]) -- the step every rank runs on its own buffer.
+template <class Sum, int W, int R, int LOW>
+__device__ __forceinline__ u32x4 subtree(const u32x4 (&x)[W])
+{
+    Sum acc;
+    acc.zero();
+    if constexpr (LOW > 1) {
+        acc.add(subtree<Sum, W, R - LOW / 2, LOW / 2>(x));
+        acc.add(subtree<Sum, W, R + LOW / 2, LOW / 2>(x));
+    }
+    acc.add(x[R]);
+    return acc.result();
+}
+
+// The extra node 0 on top: round(0 + node(W/2) + x[0]).
+template <class Sum, int W>
+__device__ __forceinline__ u32x4 whole_tree(const u32x4 (&x)[W])
+{
+    Sum acc;
+    acc.zero();
+    acc.add(subtree<Sum, W, W / 2, W / 2>(x));
+    acc.add(x[0]);
+    return acc.result();
+}
+
+template <int W>
+struct TreePtrs {
+    char *buf[W];
+    char *out[W]; // entries may be null
+};
+
+// Vectors [begin, end) of one half; SHIFT = 0 for tree a, W-1 for tree b (label l lives in
+// rank (l + SHIFT) mod W), a compile-time constant so that every pointer stays in SGPRs.
+template <class Sum, int W, int SHIFT>
+__device__ __forceinline__ void fused_half(const TreePtrs<W> &p, size_t begin, size_t end)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    for (size_t i = begin + static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < end; i += stride) {
+        u32x4 x[W];
+#pragma unroll
+        for (int l = 0; l < W; ++l) x[l] = load_vec<false>(p.buf[(l + SHIFT) % W], i);
+        const u32x4 s = whole_tree<Sum, W>(x);
+#pragma unroll
+        for (int r = 0; r < W; ++r) store_vec<false>(p.buf[r], i, s);
+#pragma unroll
+        for (int r = 0; r < W; ++r)
+            if (p.out[r] != nullptr) store_vec<false>(p.out[r], i, s);
+    }
+}
+
+template <class Sum, int W>
+__global__ void __launch_bounds__(kPhasedBlock) tree_fused_kernel(TreePtrs<W> p, size_t nvec, size_t split_vec)
+{
+    fused_half<Sum, W, 0>(p, 0, split_vec);
+    fused_half<Sum, W, W - 1>(p, split_vec, nvec);
+}
+
+template <class Sum, int W>
+static hipError_t launch_fused(void *const *bufs, void *const *outs, size_t nvec, size_t split_vec, hipStream_t stream)
+{
+    TreePtrs<W> p;
+    for (int r = 0; r < W; ++r) {
+        p.buf[r] = static_cast<char *>(bufs[r]);
+        p.out[r] = outs ? static_cast<char *>(outs[r]) : nullptr;
+    }
+    size_t grid = (nvec + kPhasedBlock - 1) / kPhasedBlock;
+    const size_t cap = static_cast<size_t>(compute_units()) * 8;
+    if (grid > cap) grid = cap;
+    if (grid == 0) grid = 1;
+    hipLaunchKernelGGL((tree_fused_kernel<Sum, W>), dim3(static_cast<unsigned>(grid)), dim3(kPhasedBlock), 0, stream, p,
+                       nvec, split_vec);
+    return hipGetLastError();
+}
+
+template <class Sum>
+static hipError_t launch_fused_world(void *const *bufs, void *const *outs, int world, size_t nvec, size_t split_vec,
+                                     hipStream_t stream)
+{
+    switch (world) {
+    case 2: return launch_fused<Sum, 2>(bufs, outs, nvec, split_vec, stream);
+    case 4: return launch_fused<Sum, 4>(bufs, outs, nvec, split_vec, stream);
+    case 8: return launch_fused<Sum, 8>(bufs, outs, nvec, split_vec, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+} // namespace tccl
+
+extern "C" int tccl_double_tree_all_reduce_fused(void *const *bufs, void *const *outs, int world, size_t numel,
+                                                 int dtype, void *stream)
+{
+    const int esize = dtype_size(dtype);
+    if (esize == 0 || bufs == nullptr) return TCCL_EINVAL;
+    if (!pow2_world(world)) return TCCL_EPOW2;
+    if (world > 8) return TCCL_EINVAL;
+    for (int r = 0; r < world; ++r) {
+        if (bufs[r] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(bufs[r]) || (outs && !aligned16(outs[r]))) return TCCL_EALIGN;
+    }
+    const size_t per_vec = kVecBytes / esize;
+    if (numel % per_vec != 0) return TCCL_EALIGN;
+    if (numel == 0) return TCCL_OK;
+    const size_t nvec = numel / per_vec;
+    const size_t split_vec = tccl_double_tree_split(numel, esize) / per_vec;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = (dtype == TCCL_BF16) ? launch_fused_world<Bf16Sum>(bufs, outs, world, nvec, split_vec, s)
+                                        : launch_fused_world<F32Sum>(bufs, outs, world, nvec, split_vec, s);
+    return hip_code(e);
+}
+
 // ------------------------------------------------------------------ recorded plans
 
 struct tccl_plan {

@@ -21,7 +21,7 @@ REPS = 10          # as in the reference
 
 def main(argv=None) -> int:
     p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    p.add_argument("op", choices=["all_reduce", "reduce_scatter", "all_gather", "double_tree", "double_tree_plan",
+    p.add_argument("op", choices=["all_reduce", "reduce_scatter", "all_gather", "double_tree", "double_tree_plan", "double_tree_fused",
                                   "two_shot"])
     p.add_argument("--world", type=int, default=8)
     p.add_argument("--max-elems", type=int, default=256 * 1024 * 1024 // 2,
@@ -47,7 +47,8 @@ def main(argv=None) -> int:
         "two_shot": (tccl_amd.two_shot_all_reduce, lambda n: (world + 3) * n * 2),
         "reduce_scatter": (tccl_amd.reduce_scatter, lambda n: (world + 1) * (n // world) * 2),
         "all_gather": (lambda t: tccl_amd.all_gather(t, world), lambda n: 2 * world * n * 2),
-        "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel()), None),
+        "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=False), None),
+        "double_tree_fused": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=True), None),
     }
     size = args.max_elems
     while size >= 2048:

@@ -73,6 +73,9 @@ def test_argument_checks_return_codes_without_launching():
     assert lib.tccl_double_tree_all_reduce(good, None, 128, 64, 0, 0, None) == -1
     assert lib.tccl_double_tree_all_reduce(good, None, 2, 60, 0, 0, None) == -2
     assert lib.tccl_double_tree_all_reduce(good, None, 2, 0, 0, 0, None) == 0
+    assert lib.tccl_double_tree_all_reduce_fused(good, None, 16, 64, 0, None) == -1
+    assert lib.tccl_double_tree_all_reduce_fused(None, None, 8, 64, 0, None) == -1
+    assert lib.tccl_double_tree_all_reduce_fused(good, None, 2, 0, 0, None) == 0
     assert lib.tccl_double_tree_plan_create(good, None, 2, 64, 0, 0, None) == -1
     assert lib.tccl_plan_launch(None, None) == -1
     assert lib.tccl_plan_destroy(None) == -1

@@ -463,10 +463,43 @@ def test_double_tree_all_ranks(world, numel, _gpu_hygiene, c_oracle):
     want = from_np_bits(outs[0])
     assert_bit_equal(want, torch_ref.double_tree_all_reduce(bufs)[0], "oracles agree")
     g = upload(_gpu_hygiene, bufs)
-    got = [tccl_amd.double_tree_all_reduce(g.tensor(r)) for r in range(world)]   # one call per rank
+    got = [tccl_amd.double_tree_all_reduce(g.tensor(r), fused=False) for r in range(world)]   # one call per rank
     for r in range(world):
         assert_bit_equal(got[r], want, f"output of rank {r}")
         assert_bit_equal(g.tensor(r), from_np_bits(final[r]), f"buffer of rank {r}")
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+@pytest.mark.parametrize("numel", [8, 24, 8 * 12_345, 65_536 * 4 + 8, 8 * 1_000_003])
+def test_double_tree_one_launch_kernel(world, maker, numel, _gpu_hygiene, c_oracle):
+    """The whole tree in one launch against the level schedule and the oracle: same outputs,
+    same final buffers, bit for bit."""
+    bufs = maker(world, numel, seed_base=300)
+    want = torch_ref.double_tree_all_reduce(bufs)[0]
+    if maker is seeded_randn:
+        _, outs = c_oracle.double_tree_all_reduce_bf16([np_bits(b) for b in bufs])
+        assert_bit_equal(from_np_bits(outs[0]), want, "oracles agree")
+    g = upload(_gpu_hygiene, bufs)
+    fused = tccl_amd.double_tree_all_reduce_world(g, fused=True)
+    for r in range(world):
+        assert_bit_equal(fused[r], want, f"one launch, output {r}")
+        assert_bit_equal(g.tensor(r), want, f"one launch, buffer {r}")
+    g2 = upload(_gpu_hygiene, bufs)
+    levels = tccl_amd.double_tree_all_reduce_world(g2, fused=False)
+    for r in range(world):
+        assert_bit_equal(levels[r], fused[r], f"schedule vs one launch, output {r}")
+
+
+def test_double_tree_one_launch_limits(_gpu_hygiene):
+    g = tccl_amd.empty_world(16, 64, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    with pytest.raises(tccl_amd.TcclError):
+        tccl_amd.double_tree_all_reduce_world(g, fused=True)          # worlds of 2, 4, 8 only
+    assert len(tccl_amd.double_tree_all_reduce_world(g)) == 16         # auto falls back to the schedule
+    lib = tccl_amd.load_library()
+    assert lib.tccl_double_tree_all_reduce_fused(g.ptr_array, None, 3, 64, 0, None) == -3
+    assert lib.tccl_double_tree_all_reduce_fused(g.ptr_array, None, 8, 60, 0, None) == -2
 
 
 def test_double_tree_fill_rank_and_second_collective(_gpu_hygiene):
