@@ -429,28 +429,29 @@ struct TreePtrs {
 
 // Vectors [begin, end) of one half; SHIFT = 0 for tree a, W-1 for tree b (label l lives in
 // rank (l + SHIFT) mod W), a compile-time constant so that every pointer stays in SGPRs.
-template <class Sum, int W, int SHIFT>
+template <class Sum, int W, int SHIFT, bool NT>
 __device__ __forceinline__ void fused_half(const TreePtrs<W> &p, size_t begin, size_t end)
 {
     const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
     for (size_t i = begin + static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < end; i += stride) {
         u32x4 x[W];
 #pragma unroll
-        for (int l = 0; l < W; ++l) x[l] = load_vec<false>(p.buf[(l + SHIFT) % W], i);
+        for (int l = 0; l < W; ++l) x[l] = load_vec<NT>(p.buf[(l + SHIFT) % W], i);
         const u32x4 s = whole_tree<Sum, W>(x);
 #pragma unroll
-        for (int r = 0; r < W; ++r) store_vec<false>(p.buf[r], i, s);
+        for (int r = 0; r < W; ++r) store_vec<NT>(p.buf[r], i, s);
 #pragma unroll
         for (int r = 0; r < W; ++r)
-            if (p.out[r] != nullptr) store_vec<false>(p.out[r], i, s);
+            if (p.out[r] != nullptr) store_vec<NT>(p.out[r], i, s);
     }
 }
 
-template <class Sum, int W>
+// NT = streaming loads and stores, for inputs too large to stay in the caches.
+template <class Sum, int W, bool NT>
 __global__ void __launch_bounds__(kPhasedBlock) tree_fused_kernel(TreePtrs<W> p, size_t nvec, size_t split_vec)
 {
-    fused_half<Sum, W, 0>(p, 0, split_vec);
-    fused_half<Sum, W, W - 1>(p, split_vec, nvec);
+    fused_half<Sum, W, 0, NT>(p, 0, split_vec);
+    fused_half<Sum, W, W - 1, NT>(p, split_vec, nvec);
 }
 
 template <class Sum, int W>
@@ -461,12 +462,20 @@ static hipError_t launch_fused(void *const *bufs, void *const *outs, size_t nvec
         p.buf[r] = static_cast<char *>(bufs[r]);
         p.out[r] = outs ? static_cast<char *>(outs[r]) : nullptr;
     }
+    // Small inputs: every lane its own vector, cached accesses.  Large inputs (beyond the caches):
+    // one workgroup per compute unit walking the range, streaming accesses -- the shape that
+    // measured best for write-heavy streams on this GPU.
+    const bool big = nvec * kVecBytes * W >= (static_cast<size_t>(256) << 20);
     size_t grid = (nvec + kPhasedBlock - 1) / kPhasedBlock;
-    const size_t cap = static_cast<size_t>(compute_units()) * 8;
+    const size_t cap = static_cast<size_t>(compute_units()) * (big ? 1 : 8);
     if (grid > cap) grid = cap;
     if (grid == 0) grid = 1;
-    hipLaunchKernelGGL((tree_fused_kernel<Sum, W>), dim3(static_cast<unsigned>(grid)), dim3(kPhasedBlock), 0, stream, p,
-                       nvec, split_vec);
+    if (big)
+        hipLaunchKernelGGL((tree_fused_kernel<Sum, W, true>), dim3(static_cast<unsigned>(grid)), dim3(kPhasedBlock), 0,
+                           stream, p, nvec, split_vec);
+    else
+        hipLaunchKernelGGL((tree_fused_kernel<Sum, W, false>), dim3(static_cast<unsigned>(grid)), dim3(kPhasedBlock), 0,
+                           stream, p, nvec, split_vec);
     return hipGetLastError();
 }
 
