@@ -18,8 +18,14 @@ from .symm import SymmGroup, SymmHandle, rendezvous
 _SUM_DTYPES = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}
 
 
-def _stream() -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream(device: Optional[torch.device] = None) -> ctypes.c_void_p:
+    """torch's current stream on the tensor's device as a raw ``hipStream_t``."""
+    if _raw_stream is not None and device is not None and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))       # no Stream object is built
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
 def _sum_dtype(tensor: torch.Tensor) -> int:
@@ -49,7 +55,7 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCfg] =
     output = torch.empty_like(tensor)
     lib = _lib.load()
     rc = lib.tccl_all_reduce_sum_ex(symm.buffer_ptrs_host, symm.world_size, output.data_ptr(), tensor.numel(),
-                                    dtype, _stream(), _cfg_ptr(cfg))
+                                    dtype, _stream(tensor.device), _cfg_ptr(cfg))
     _lib.check("tccl_all_reduce_sum", rc)
     return output
 
@@ -68,7 +74,7 @@ def one_shot_reduce_scatter(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCf
     output = torch.empty_like(flat[per_rank * rank:per_rank * (rank + 1)])
     lib = _lib.load()
     rc = lib.tccl_reduce_scatter_sum_ex(symm.buffer_ptrs_host, world, rank, output.data_ptr(), tensor.numel(),
-                                        dtype, _stream(), _cfg_ptr(cfg))
+                                        dtype, _stream(tensor.device), _cfg_ptr(cfg))
     _lib.check("tccl_reduce_scatter_sum", rc)
     return output
 
@@ -88,8 +94,8 @@ def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, 
     assert nbytes % 16 == 0, "The number of elements must be 128-bit aligned."
     output = torch.empty((world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
     lib = _lib.load()
-    rc = lib.tccl_all_gather_ex(symm.buffer_ptrs_host, world_size, output.data_ptr(), nbytes, _stream(),
-                                _cfg_ptr(cfg))
+    rc = lib.tccl_all_gather_ex(symm.buffer_ptrs_host, world_size, output.data_ptr(), nbytes,
+                                _stream(tensor.device), _cfg_ptr(cfg))
     _lib.check("tccl_all_gather", rc)
     return output
 
@@ -110,7 +116,7 @@ def two_shot_all_reduce(tensor: torch.Tensor) -> torch.Tensor:
     assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
     per_rank = tensor.numel() // world
     lib = _lib.load()
-    stream = _stream()
+    stream = _stream(tensor.device)
     shares = torch.empty((world, per_rank), dtype=tensor.dtype, device=tensor.device)
     for r in range(world):
         rc = lib.tccl_reduce_scatter_sum(symm.buffer_ptrs_host, world, r, shares[r].data_ptr(), tensor.numel(),
@@ -155,11 +161,11 @@ def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tenso
         fused = group.world_size <= 8 and numel * like.element_size() <= FUSED_TREE_MAX_BYTES
     if fused:
         rc = lib.tccl_double_tree_all_reduce_fused(group.ptr_array, out_ptrs, group.world_size, numel, dtype,
-                                                   _stream())
+                                                   _stream(like.device))
         _lib.check("tccl_double_tree_all_reduce_fused", rc)
     else:
         rc = lib.tccl_double_tree_all_reduce(group.ptr_array, out_ptrs, group.world_size, numel, dtype, chunk_elems,
-                                             _stream())
+                                             _stream(like.device))
         _lib.check("tccl_double_tree_all_reduce", rc)
     return outputs
 
@@ -232,7 +238,7 @@ class DoubleTreePlan:
     def run(self) -> List[torch.Tensor]:
         if not self._plan:
             raise RuntimeError("plan has been closed")
-        _lib.check("tccl_plan_launch", _lib.load().tccl_plan_launch(self._plan, _stream()))
+        _lib.check("tccl_plan_launch", _lib.load().tccl_plan_launch(self._plan, _stream(self.outputs[0].device)))
         return self.outputs
 
     def close(self) -> None:
