@@ -62,6 +62,25 @@ def build(verbose: bool = False, jobs: int = 4) -> str:
     return LIB_PATH
 
 
+def build_c_client(verbose: bool = False) -> str:
+    """Compile the plain C client of the library (tests/c_client) next to its source."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "c_client", "c_abi_client.c")
+    out_dir = os.path.join(root, "tests", "c_client", "build")
+    os.makedirs(out_dir, exist_ok=True)
+    exe = os.path.join(out_dir, "c_abi_client")
+    cmd = [_hipcc(), "-x", "c", "-std=c11", "-O1", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(root, "include"),
+           "-I", "/opt/rocm/include", src, "-L", HERE, "-ltccl_amd", "-L", "/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath," + HERE, "-Wl,-rpath,/opt/rocm/lib", "-o", exe]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building the C client failed:\n{proc.stdout}\n{proc.stderr}")
+    if verbose:
+        print(f"built {exe}")
+    return exe
+
+
 if __name__ == "__main__":
     build(verbose=True)
+    build_c_client(verbose=True)
     sys.exit(0)

@@ -98,3 +98,37 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    """sizeof/offsetof of the two structs that cross the ABI, as gcc sees the header, against
+    the ctypes mirrors."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "tccl_amd.h"\n'
+        'int main(void) {\n'
+        '  printf("%zu %zu %zu %zu %zu %zu\\n", sizeof(tccl_launch_cfg), offsetof(tccl_launch_cfg, block),\n'
+        '         offsetof(tccl_launch_cfg, unroll), offsetof(tccl_launch_cfg, grid),\n'
+        '         offsetof(tccl_launch_cfg, tile_iters), offsetof(tccl_launch_cfg, flags));\n'
+        '  printf("%zu %zu %zu %zu %zu\\n", sizeof(tccl_node_job), offsetof(tccl_node_job, src),\n'
+        '         offsetof(tccl_node_job, dst), offsetof(tccl_node_job, numel), offsetof(tccl_node_job, is_copy));\n'
+        '  printf("%d %d %d %d %d %d\\n", TCCL_ABI_VERSION, TCCL_MAX_WORLD, TCCL_MAX_JOBS, TCCL_BF16, TCCL_F32,\n'
+        '         TCCL_CFG_PHASED);\n'
+        '  return 0;\n}\n')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    lines = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    cfg = [int(x) for x in lines[0].split()]
+    job = [int(x) for x in lines[1].split()]
+    consts = [int(x) for x in lines[2].split()]
+    C = _lib.LaunchCfg
+    assert cfg == [ctypes.sizeof(C), C.block.offset, C.unroll.offset, C.grid.offset, C.tile_iters.offset,
+                   C.flags.offset]
+    J = _lib.NodeJob
+    assert job == [ctypes.sizeof(J), J.src.offset, J.dst.offset, J.numel.offset, J.is_copy.offset]
+    assert consts == [_lib.ABI_VERSION, _lib.MAX_WORLD, _lib.MAX_JOBS, _lib.TCCL_BF16, _lib.TCCL_F32,
+                      _lib.CFG_PHASED]

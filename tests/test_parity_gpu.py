@@ -583,3 +583,20 @@ def test_double_tree_config5_properties(_gpu_hygiene, c_oracle):
         w = from_np_bits(want[0])
         assert_bit_equal(outs[0][lo:lo + n], w[:n], f"tree a window at {lo}")
         assert_bit_equal(outs[0][half + lo:half + lo + n], w[n:], f"tree b window at {lo}")
+
+
+# ------------------------------------------------------------------ a client without Python
+
+def test_plain_c_client():
+    """tests/c_client/c_abi_client.c: hipMalloc'd buffers and the C entry points only (no
+    torch anywhere in the process), built by `python -m tccl_amd.build`."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "c_client", "build", "c_abi_client")
+    assert os.path.exists(exe), "C client not built: run `python -m tccl_amd.build`"
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = os.path.join(root, "tccl_amd") + os.pathsep + env.get("LD_LIBRARY_PATH", "")
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=120, env=env)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "c client ok" in proc.stdout
