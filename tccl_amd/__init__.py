@@ -6,7 +6,7 @@ from ._lib import LaunchCfg, TcclError, load as load_library
 from .collectives import (DoubleTreePlan, all_gather, all_reduce, double_tree_all_reduce, double_tree_all_reduce_world, one_shot_all_gather,
                           one_shot_all_reduce, one_shot_reduce_scatter, reduce_scatter, two_shot_all_reduce)
 from .symm import SymmGroup, SymmHandle, empty_world, register, rendezvous, unregister
-from . import tree
+from . import spmd, tree
 from .tree import build_double_tree, build_tree, get_parents_and_children
 
 __all__ = [
@@ -14,5 +14,5 @@ __all__ = [
     "one_shot_all_reduce", "one_shot_reduce_scatter", "one_shot_all_gather", "double_tree_all_reduce",
     "double_tree_all_reduce_world", "DoubleTreePlan", "reduce_scatter", "all_gather", "two_shot_all_reduce", "all_reduce",
     "SymmGroup", "SymmHandle", "empty_world", "register", "rendezvous", "unregister",
-    "tree", "build_tree", "build_double_tree", "get_parents_and_children",
+    "spmd", "tree", "build_tree", "build_double_tree", "get_parents_and_children",
 ]

@@ -12,7 +12,7 @@ from typing import List, Optional
 
 import torch
 
-from . import _lib
+from . import _lib, spmd
 from .symm import SymmGroup, SymmHandle, rendezvous
 
 _SUM_DTYPES = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}
@@ -51,12 +51,13 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCfg] =
     is accumulated in fp32 in rank order and rounded once."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
-    symm = rendezvous(tensor)
-    output = torch.empty_like(tensor)
     lib = _lib.load()
-    rc = lib.tccl_all_reduce_sum_ex(symm.buffer_ptrs_host, symm.world_size, output.data_ptr(), tensor.numel(),
-                                    dtype, _stream(tensor.device), _cfg_ptr(cfg))
-    _lib.check("tccl_all_reduce_sum", rc)
+    with spmd.collective():
+        symm = rendezvous(tensor)
+        output = torch.empty_like(tensor)
+        rc = lib.tccl_all_reduce_sum_ex(symm.buffer_ptrs_host, symm.world_size, output.data_ptr(), tensor.numel(),
+                                        dtype, _stream(tensor.device), _cfg_ptr(cfg))
+        _lib.check("tccl_all_reduce_sum", rc)
     return output
 
 
@@ -66,16 +67,17 @@ def one_shot_reduce_scatter(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCf
     Mirrors ``one_shot_reduce_scatter`` (triton_reduce_scatter.py:95-127); rank and world
     size come from the handle (the reference reads module globals, :103-113)."""
     dtype = _sum_dtype(tensor)
-    symm = rendezvous(tensor)
-    world, rank = symm.world_size, symm.rank
-    assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
-    per_rank = tensor.numel() // world
-    flat = tensor.reshape(-1)
-    output = torch.empty_like(flat[per_rank * rank:per_rank * (rank + 1)])
     lib = _lib.load()
-    rc = lib.tccl_reduce_scatter_sum_ex(symm.buffer_ptrs_host, world, rank, output.data_ptr(), tensor.numel(),
-                                        dtype, _stream(tensor.device), _cfg_ptr(cfg))
-    _lib.check("tccl_reduce_scatter_sum", rc)
+    with spmd.collective():
+        symm = rendezvous(tensor)
+        world, rank = symm.world_size, symm.rank
+        assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
+        per_rank = tensor.numel() // world
+        flat = tensor.reshape(-1)
+        output = torch.empty_like(flat[per_rank * rank:per_rank * (rank + 1)])
+        rc = lib.tccl_reduce_scatter_sum_ex(symm.buffer_ptrs_host, world, rank, output.data_ptr(), tensor.numel(),
+                                            dtype, _stream(tensor.device), _cfg_ptr(cfg))
+        _lib.check("tccl_reduce_scatter_sum", rc)
     return output
 
 
@@ -86,17 +88,18 @@ def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, 
     Mirrors ``one_shot_all_gather(tensor, world_size)`` (triton_all_gather.py:66-95).  Any
     dtype is copied bit for bit (the reference asserts bfloat16, :72, though its copy is
     typeless); the byte count per rank must be a multiple of 16 (:73-75)."""
-    symm = rendezvous(tensor)
-    if world_size is None:
-        world_size = symm.world_size
-    assert world_size == symm.world_size, "world_size does not match the tensor's symmetric group"
     nbytes = tensor.numel() * tensor.element_size()
     assert nbytes % 16 == 0, "The number of elements must be 128-bit aligned."
-    output = torch.empty((world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
     lib = _lib.load()
-    rc = lib.tccl_all_gather_ex(symm.buffer_ptrs_host, world_size, output.data_ptr(), nbytes,
-                                _stream(tensor.device), _cfg_ptr(cfg))
-    _lib.check("tccl_all_gather", rc)
+    with spmd.collective():
+        symm = rendezvous(tensor)
+        if world_size is None:
+            world_size = symm.world_size
+        assert world_size == symm.world_size, "world_size does not match the tensor's symmetric group"
+        output = torch.empty((world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
+        rc = lib.tccl_all_gather_ex(symm.buffer_ptrs_host, world_size, output.data_ptr(), nbytes,
+                                    _stream(tensor.device), _cfg_ptr(cfg))
+        _lib.check("tccl_all_gather", rc)
     return output
 
 
@@ -111,21 +114,22 @@ def two_shot_all_reduce(tensor: torch.Tensor) -> torch.Tensor:
     (triton_reduce_scatter.py:101-104).  On several GPUs this moves (W-1)/W of a buffer per
     direction over the links instead of (W-1) whole buffers."""
     dtype = _sum_dtype(tensor)
-    symm = rendezvous(tensor)
-    world = symm.world_size
-    assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
-    per_rank = tensor.numel() // world
     lib = _lib.load()
     stream = _stream(tensor.device)
-    shares = torch.empty((world, per_rank), dtype=tensor.dtype, device=tensor.device)
-    for r in range(world):
-        rc = lib.tccl_reduce_scatter_sum(symm.buffer_ptrs_host, world, r, shares[r].data_ptr(), tensor.numel(),
-                                         dtype, stream)
-        _lib.check("tccl_reduce_scatter_sum", rc)
-    share_ptrs = _lib.ptr_array([int(shares[r].data_ptr()) for r in range(world)])
-    output = torch.empty_like(tensor)
-    rc = lib.tccl_all_gather(share_ptrs, world, output.data_ptr(), per_rank * tensor.element_size(), stream)
-    _lib.check("tccl_all_gather", rc)
+    with spmd.collective():
+        symm = rendezvous(tensor)
+        world = symm.world_size
+        assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
+        per_rank = tensor.numel() // world
+        shares = torch.empty((world, per_rank), dtype=tensor.dtype, device=tensor.device)
+        output = torch.empty_like(tensor)
+        for r in range(world):
+            rc = lib.tccl_reduce_scatter_sum(symm.buffer_ptrs_host, world, r, shares[r].data_ptr(), tensor.numel(),
+                                             dtype, stream)
+            _lib.check("tccl_reduce_scatter_sum", rc)
+        share_ptrs = _lib.ptr_array([int(shares[r].data_ptr()) for r in range(world)])
+        rc = lib.tccl_all_gather(share_ptrs, world, output.data_ptr(), per_rank * tensor.element_size(), stream)
+        _lib.check("tccl_all_gather", rc)
     return output
 
 
@@ -190,6 +194,16 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
     one-launch kernel up to ``FUSED_TREE_MAX_BYTES`` per buffer, the level schedule above."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
+    if spmd.current_rank() is not None:
+        # W rank threads arrive together: one of them runs the collective for everybody,
+        # the others pick their output up once it has been enqueued.
+        with spmd.collective() as turn:
+            symm = rendezvous(tensor)
+            group = symm.group
+            if turn.first:
+                group.pending_outputs = dict(enumerate(
+                    _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems, fused)))
+        return group.pending_outputs[symm.rank]
     symm = rendezvous(tensor)
     group = symm.group
     pending = group.pending_outputs.pop(symm.rank, None)
