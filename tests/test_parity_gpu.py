@@ -151,6 +151,27 @@ def test_phased_and_streaming_kernels_agree_at_headline_size(_gpu_hygiene, c_ora
         assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0), cfg=cfg), want, f"flags={flags}")
 
 
+@pytest.mark.parametrize("world,mib", [(8, 4), (8, 64), (5, 64), (4, 64), (3, 96), (2, 48), (1, 48), (1, 4)])
+def test_all_reduce_around_dispatch_thresholds(world, mib, _gpu_hygiene, c_oracle):
+    """Sizes one vector below, at, one vector above and raggedly above every size at which
+    the library changes kernel or launch plan (grid-stride -> phased at 4 MiB of output, one
+    resident wave of tiles at 64 MiB, the single-launch rule for few sources at 48/96 MiB)."""
+    base = (mib << 20) // 2
+    top = base + 8 * 1025 + 3
+    torch.manual_seed(world * 1000 + mib)
+    first = torch.randn(top, dtype=torch.bfloat16)
+    bufs = [first.roll(r * 104_729) for r in range(world)]
+    g = upload(_gpu_hygiene, bufs)
+    lib = tccl_amd.load_library()
+    out = torch.empty(top + 64, dtype=torch.bfloat16, device=DEV)
+    for numel in (base - 8, base, base + 8, base + 8 * 1025 + 3):
+        out.fill_(9.0)
+        assert lib.tccl_all_reduce_sum(g.ptr_array, world, out.data_ptr(), numel, _lib.TCCL_BF16, stream()) == 0
+        want = oracle_sum(c_oracle, [b[:numel].contiguous() for b in bufs])
+        assert_bit_equal(out[:numel], want, f"W={world} numel={numel}")
+        assert out[numel:numel + 64].eq(9.0).all().item(), "wrote past the end"
+
+
 def test_all_reduce_order_and_single_rounding(_gpu_hygiene):
     """fp32 accumulation in rank order: [2^24, 1 x6, -2^24] -> 0; ones first -> 6;
     1 + 2^-8 + 2^-8 -> 1 + 2^-7 (a bf16-stepwise sum would give 1)."""
