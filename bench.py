@@ -31,10 +31,10 @@ BYTES_PER_BUF = 64 << 20
 LAT_BYTES_PER_BUF = 1 << 20
 
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs of this script
-# (FETCH_SIZE 262,353.78 KiB and WRITE_SIZE 65,536.00 KiB per dispatch), each scaled by what
+# (FETCH_SIZE 262,354.07 KiB and WRITE_SIZE 65,536.00 KiB per dispatch), each scaled by what
 # the same counter reads for the 256 MiB plain copy of --calibrate-copy (factors 1.99959 and
-# 1.00000): 524,601 KiB fetched + 65,536 KiB written.
-MEASURED_TRAFFIC_BYTES = 604_300_375
+# 0.99996): 524,600 KiB fetched + 65,533 KiB written.
+MEASURED_TRAFFIC_BYTES = 604_296_372
 
 
 def parse_args():
