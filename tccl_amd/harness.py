@@ -26,6 +26,9 @@ def main(argv=None) -> int:
     p.add_argument("--world", type=int, default=8)
     p.add_argument("--max-elems", type=int, default=256 * 1024 * 1024 // 2,
                    help="largest element count per rank (bf16); halved down to 2,048")
+    p.add_argument("--compare", action="store_true",
+                   help="also time the same operation written with torch's own GPU kernels, as the second "
+                        "line per size (the place the reference gives to NCCL)")
     args = p.parse_args(argv)
 
     import torch
@@ -50,6 +53,22 @@ def main(argv=None) -> int:
         "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=False), None),
         "double_tree_fused": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=True), None),
     }
+
+    def torch_eager(view):
+        """The operation with torch's stock kernels on the same buffers (fp32 accumulate)."""
+        n = view.numel()
+        srcs = [group.tensor(r)[:n] for r in range(world)]
+        if args.op == "all_gather":
+            return torch.stack(srcs)
+        if args.op == "reduce_scatter":
+            per = n // world
+            r = min(3, world - 1)
+            srcs = [b[r * per:(r + 1) * per] for b in srcs]
+        acc = srcs[0].float()
+        for b in srcs[1:]:
+            acc += b
+        return acc.to(view.dtype)
+
     size = args.max_elems
     while size >= 2048:
         view = tensor[:size]
@@ -73,6 +92,16 @@ def main(argv=None) -> int:
         else:
             line += f"  ({per_call_ms * 1e3:.1f} us)"
         print(line, flush=True)
+        if args.compare:
+            torch_eager(view)
+            lib.tccl_event_record(start, stream)
+            for _ in range(REPS):
+                torch_eager(view)
+            lib.tccl_event_record(stop, stream)
+            lib.tccl_event_synchronize(stop)
+            lib.tccl_event_elapsed_ms(start, stop, ctypes.byref(ms))
+            t_ms = ms.value / REPS
+            print(f"torch {size * 2} {size * 2 / t_ms / 1e6:.3f} GB/s  ({t_ms * 1e3:.1f} us)", flush=True)
         size //= 2
     tccl_amd.unregister(group)
     return 0
