@@ -277,6 +277,48 @@ def test_launches_follow_the_current_stream(_gpu_hygiene, c_oracle):
     assert torch.equal(doubled.cpu(), want.float() * 2)
 
 
+def test_entry_points_can_be_captured_in_a_graph(_gpu_hygiene, c_oracle):
+    """The entry points neither allocate nor synchronise, so a caller can record them into a
+    HIP graph of its own (here through torch.cuda.graph) and replay it.  Replayed several
+    times with new inputs and eager work in between; every replay is checked."""
+    world, numel = 8, 8 * 8 * 20_001
+    g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    lib = tccl_amd.load_library()
+    out = torch.empty(numel, dtype=torch.bfloat16, device=DEV)
+    share = torch.empty(numel // world, dtype=torch.bfloat16, device=DEV)
+    gathered = torch.empty((world, numel), dtype=torch.bfloat16, device=DEV)
+
+    def enqueue():
+        s = stream()
+        assert lib.tccl_all_reduce_sum(g.ptr_array, world, out.data_ptr(), numel, _lib.TCCL_BF16, s) == 0
+        assert lib.tccl_reduce_scatter_sum(g.ptr_array, world, 5, share.data_ptr(), numel, _lib.TCCL_BF16, s) == 0
+        assert lib.tccl_all_gather(g.ptr_array, world, gathered.data_ptr(), numel * 2, s) == 0
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue()                                  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue()
+    per = numel // world
+    for rep in range(4):
+        bufs = seeded_randn(world, numel, seed_base=500 + 10 * rep)
+        for r in range(world):
+            g.tensor(r).copy_(bufs[r])
+        out.zero_(), share.zero_(), gathered.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle_sum(c_oracle, bufs)
+        assert_bit_equal(out, want, f"replay {rep} all-reduce")
+        assert_bit_equal(share, want[5 * per:6 * per], f"replay {rep} reduce-scatter")
+        assert_bit_equal(gathered, torch.stack(bufs), f"replay {rep} all-gather")
+        assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0)), want, f"eager after replay {rep}")
+
+
 # ------------------------------------------------------------------ reduce-scatter
 
 @pytest.mark.parametrize("world", [2, 4, 8])
