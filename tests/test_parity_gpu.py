@@ -277,6 +277,49 @@ def test_launches_follow_the_current_stream(_gpu_hygiene, c_oracle):
     assert torch.equal(doubled.cpu(), want.float() * 2)
 
 
+def test_concurrent_callers_on_their_own_streams(_gpu_hygiene, c_oracle):
+    """The library keeps no state between calls: four host threads, each with its own group
+    and its own stream, call every operation at the same time."""
+    import threading
+    world, numel, threads = 4, 8 * 4 * 30_011, 4
+    inputs = [seeded_randn(world, numel, seed_base=900 + 10 * t) for t in range(threads)]
+    groups = [upload(_gpu_hygiene, inputs[t]) for t in range(threads)]
+    torch.cuda.synchronize()
+    results, errors = [None] * threads, []
+
+    def work(t):
+        try:
+            torch.cuda.set_device(0)
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                acc = []
+                for _ in range(20):
+                    ar = tccl_amd.one_shot_all_reduce(groups[t].tensor(0))
+                    rs = tccl_amd.reduce_scatter(groups[t].tensor(t % world))
+                    ag = tccl_amd.all_gather(groups[t].tensor(0), world)
+                    ts = tccl_amd.two_shot_all_reduce(groups[t].tensor(1))
+                    acc.append((ar, rs, ag, ts))
+                s.synchronize()
+            results[t] = acc
+        except BaseException as e:       # noqa: BLE001 -- reported below
+            errors.append(e)
+
+    pool = [threading.Thread(target=work, args=(t,)) for t in range(threads)]
+    for p in pool:
+        p.start()
+    for p in pool:
+        p.join()
+    assert not errors, errors
+    per = numel // world
+    for t in range(threads):
+        want = oracle_sum(c_oracle, inputs[t])
+        for ar, rs, ag, ts in results[t][::7]:
+            assert_bit_equal(ar, want, f"thread {t} all-reduce")
+            assert_bit_equal(rs, want[(t % world) * per:(t % world + 1) * per], f"thread {t} reduce-scatter")
+            assert_bit_equal(ag, torch.stack(inputs[t]), f"thread {t} all-gather")
+            assert_bit_equal(ts, want, f"thread {t} two-shot")
+
+
 def test_entry_points_can_be_captured_in_a_graph(_gpu_hygiene, c_oracle):
     """The entry points neither allocate nor synchronise, so a caller can record them into a
     HIP graph of its own (here through torch.cuda.graph) and replay it.  Replayed several
