@@ -362,6 +362,51 @@ def test_entry_points_can_be_captured_in_a_graph(_gpu_hygiene, c_oracle):
         assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0)), want, f"eager after replay {rep}")
 
 
+def test_buffers_larger_than_4_gib(_gpu_hygiene, c_oracle):
+    """Offsets beyond 2^32 bytes inside ONE buffer: W=2 all-reduce over 2^31 + 98,760 bf16
+    elements (4 GiB + 193 KiB per buffer), all-gather of the same rows, and a two-destination
+    copy step.  Checked on the GPU in slices (with two sources the contract is exactly
+    round(a + b)), and against the C oracle on windows around the 4 GiB mark and the end."""
+    numel = (1 << 31) + 8 * 12_345
+    g = tccl_amd.empty_world(2, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    step = 1 << 28
+    for r in range(2):
+        gen = torch.Generator(device=DEV).manual_seed(40 + r)
+        for lo in range(0, numel, step):
+            n = min(step, numel - lo)
+            g.tensor(r)[lo:lo + n].copy_(torch.randn(n, dtype=torch.float32, device=DEV, generator=gen))
+    a, b = g.tensor(0), g.tensor(1)
+    out = tccl_amd.one_shot_all_reduce(a)
+    for lo in range(0, numel, step):
+        n = min(step, numel - lo)
+        want = (a[lo:lo + n].float() + b[lo:lo + n].float()).to(torch.bfloat16)
+        assert torch.equal(out[lo:lo + n].view(torch.int16), want.view(torch.int16)), f"slice at {lo}"
+    for lo, n in (((1 << 31) - 4096, 8192), (numel - 8 * 1000, 8 * 1000), (0, 4096)):
+        want = oracle_sum(c_oracle, [a[lo:lo + n].cpu(), b[lo:lo + n].cpu()])
+        assert_bit_equal(out[lo:lo + n], want, f"window at {lo}")
+    del out
+    gathered = tccl_amd.all_gather(a, 2)
+    assert torch.equal(gathered[0].view(torch.int16), a.view(torch.int16))
+    assert torch.equal(gathered[1].view(torch.int16), b.view(torch.int16))
+    del gathered
+    torch.cuda.empty_cache()
+    d0 = torch.empty_like(a)
+    d1 = torch.empty_like(a)
+    rc = tccl_amd.load_library().tccl_tree_copy_step(b.data_ptr(), d0.data_ptr(), d1.data_ptr(), numel * 2, stream())
+    assert rc == 0
+    assert torch.equal(d0.view(torch.int16), b.view(torch.int16))
+    assert torch.equal(d1.view(torch.int16), b.view(torch.int16))
+    # in-place tree reduce step over the whole 4 GiB+ range: own <- 0 + child + own
+    rc = tccl_amd.load_library().tccl_tree_reduce_step(d0.data_ptr(), a.data_ptr(), None, d0.data_ptr(), numel,
+                                                       _lib.TCCL_BF16, stream())
+    assert rc == 0
+    for lo in range(0, numel, step):
+        n = min(step, numel - lo)
+        want = (a[lo:lo + n].float() + b[lo:lo + n].float()).to(torch.bfloat16)
+        assert torch.equal(d0[lo:lo + n].view(torch.int16), want.view(torch.int16)), f"tree step slice at {lo}"
+
+
 # ------------------------------------------------------------------ reduce-scatter
 
 @pytest.mark.parametrize("world", [2, 4, 8])
