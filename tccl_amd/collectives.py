@@ -43,25 +43,34 @@ def _cfg_ptr(cfg: Optional[_lib.LaunchCfg]):
     return ctypes.byref(cfg) if cfg is not None else None
 
 
-def one_shot_all_reduce(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
+def _check_out(out: torch.Tensor, shape, like: torch.Tensor) -> torch.Tensor:
+    if tuple(out.shape) != tuple(shape) or out.dtype != like.dtype or out.device != like.device \
+            or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous {like.dtype} tensor of shape {tuple(shape)} on {like.device}")
+    return out
+
+
+def one_shot_all_reduce(tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+                        cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
     """Sum of all ranks' buffers over ``tensor.numel()`` elements.
 
     Mirrors ``one_shot_all_reduce`` (triton_one_shot_all_reduce_no_128.py:67-96): same
-    dtype and alignment assertions (:73-76), a fresh ``empty_like`` output (:83).  The sum
-    is accumulated in fp32 in rank order and rounded once."""
+    dtype and alignment assertions (:73-76), a fresh ``empty_like`` output (:83) unless the
+    caller passes ``out``.  The sum is accumulated in fp32 in rank order and rounded once."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
     lib = _lib.load()
     with spmd.collective():
         symm = rendezvous(tensor)
-        output = torch.empty_like(tensor)
+        output = torch.empty_like(tensor) if out is None else _check_out(out, tensor.shape, tensor)
         rc = lib.tccl_all_reduce_sum_ex(symm.buffer_ptrs_host, symm.world_size, output.data_ptr(), tensor.numel(),
                                         dtype, _stream(tensor.device), _cfg_ptr(cfg))
         _lib.check("tccl_all_reduce_sum", rc)
     return output
 
 
-def one_shot_reduce_scatter(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
+def one_shot_reduce_scatter(tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+                            cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
     """This rank's 1/W share of the sum: elements ``[rank*P, (rank+1)*P)``, ``P = numel // W``.
 
     Mirrors ``one_shot_reduce_scatter`` (triton_reduce_scatter.py:95-127); rank and world
@@ -73,8 +82,10 @@ def one_shot_reduce_scatter(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCf
         world, rank = symm.world_size, symm.rank
         assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
         per_rank = tensor.numel() // world
-        flat = tensor.reshape(-1)
-        output = torch.empty_like(flat[per_rank * rank:per_rank * (rank + 1)])
+        if out is None:
+            output = torch.empty((per_rank,), dtype=tensor.dtype, device=tensor.device)
+        else:
+            output = _check_out(out, (per_rank,), tensor)
         rc = lib.tccl_reduce_scatter_sum_ex(symm.buffer_ptrs_host, world, rank, output.data_ptr(), tensor.numel(),
                                             dtype, _stream(tensor.device), _cfg_ptr(cfg))
         _lib.check("tccl_reduce_scatter_sum", rc)
@@ -82,7 +93,7 @@ def one_shot_reduce_scatter(tensor: torch.Tensor, *, cfg: Optional[_lib.LaunchCf
 
 
 def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, *,
-                        cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
+                        out: Optional[torch.Tensor] = None, cfg: Optional[_lib.LaunchCfg] = None) -> torch.Tensor:
     """``[W, *tensor.shape]`` tensor whose row i is a copy of rank i's buffer.
 
     Mirrors ``one_shot_all_gather(tensor, world_size)`` (triton_all_gather.py:66-95).  Any
@@ -96,7 +107,10 @@ def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, 
         if world_size is None:
             world_size = symm.world_size
         assert world_size == symm.world_size, "world_size does not match the tensor's symmetric group"
-        output = torch.empty((world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
+        if out is None:
+            output = torch.empty((world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
+        else:
+            output = _check_out(out, (world_size, *tensor.shape), tensor)
         rc = lib.tccl_all_gather_ex(symm.buffer_ptrs_host, world_size, output.data_ptr(), nbytes,
                                     _stream(tensor.device), _cfg_ptr(cfg))
         _lib.check("tccl_all_gather", rc)

@@ -277,6 +277,27 @@ def test_launches_follow_the_current_stream(_gpu_hygiene, c_oracle):
     assert torch.equal(doubled.cpu(), want.float() * 2)
 
 
+def test_caller_provided_outputs(_gpu_hygiene, c_oracle):
+    world, numel = 4, 8 * 4 * 5_003
+    bufs = seeded_randn(world, numel, seed_base=61)
+    g = upload(_gpu_hygiene, bufs)
+    want = oracle_sum(c_oracle, bufs)
+    per = numel // world
+    out = torch.empty(numel, dtype=torch.bfloat16, device=DEV)
+    share = torch.empty(per, dtype=torch.bfloat16, device=DEV)
+    rows = torch.empty((world, numel), dtype=torch.bfloat16, device=DEV)
+    assert tccl_amd.one_shot_all_reduce(g.tensor(0), out=out) is out
+    assert tccl_amd.reduce_scatter(g.tensor(2), out=share) is share
+    assert tccl_amd.all_gather(g.tensor(0), world, out=rows) is rows
+    assert_bit_equal(out, want, "all-reduce into out")
+    assert_bit_equal(share, want[2 * per:3 * per], "reduce-scatter into out")
+    assert_bit_equal(rows, torch.stack(bufs), "all-gather into out")
+    for bad in (torch.empty(numel + 8, dtype=torch.bfloat16, device=DEV), torch.empty(numel, dtype=torch.float32, device=DEV),
+                torch.empty(2 * numel, dtype=torch.bfloat16, device=DEV)[::2]):
+        with pytest.raises(ValueError, match="out must be"):
+            tccl_amd.one_shot_all_reduce(g.tensor(0), out=bad)
+
+
 def test_concurrent_callers_on_their_own_streams(_gpu_hygiene, c_oracle):
     """The library keeps no state between calls: four host threads, each with its own group
     and its own stream, call every operation at the same time."""
