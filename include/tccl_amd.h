@@ -10,8 +10,9 @@
  *   - plain C: pointers and sizes only, no torch types.
  *   - every device pointer must be 16-byte aligned; `stream` is a hipStream_t passed as
  *     void* (NULL = the null stream).
- *   - calls are asynchronous on `stream`, allocate nothing, never synchronise and never
- *     throw; the return value is TCCL_OK or a negative code (tccl_error_string()).
+ *   - calls are asynchronous on `stream`, allocate no device memory, never synchronise and
+ *     never throw; the return value is TCCL_OK or a negative code (tccl_error_string()).
+ *     Every launching entry point can be recorded into a caller's HIP graph.
  *   - ordering between virtual ranks and between tree levels is stream order; this
  *     replaces the reference's signal-pad barrier (triton_barrier.py:39-142) and its
  *     wait/send flags (triton_double_tree_allreduce.py:175-225).
@@ -124,7 +125,10 @@ int tccl_tree_copy_step(const void *src, void *dst0, void *dst1, size_t bytes, v
 
 /* A batch of independent node steps in ONE launch (all nodes of one tree level, both
  * trees).  No counterpart in the reference, where each rank's kernel does its own step;
- * on one GPU the steps of a level are independent and share a launch. */
+ * on one GPU the steps of a level are independent and share a launch.  No job may write
+ * what another job of the same batch reads or writes.  Reduce steps are worked in tiles of
+ * at most 32 KiB (read and reduce the tile, then write it); a batch of copy steps only is
+ * walked job after job by one workgroup per compute unit. */
 typedef struct {
     const void *src[3]; /* reduce: child0, child1, own (NULL = absent); copy: src[0] only */
     void *dst[2];       /* dst[1] may be NULL */
