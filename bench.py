@@ -190,6 +190,13 @@ def main():
     lat_numel = LAT_BYTES_PER_BUF // 2
     small = mine[:lat_numel]
     p50_us, p99_us = latency_p50_us(torch, lib, lambda: tccl_amd.one_shot_all_reduce(small))
+    # the same launch through the C entry point alone (output allocated once, no wrapper work)
+    small_out = torch.empty_like(small)
+    raw_stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    c_call = lambda: lib.tccl_all_reduce_sum(group.ptr_array, WORLD, small_out.data_ptr(), lat_numel, 0, raw_stream)
+    p50_c_us, _ = latency_p50_us(torch, lib, c_call)
+    # and what one wrapper call costs end to end when calls are issued back to back
+    back_wall_ms, back_dev_ms = time_steps(torch, lib, lambda: tccl_amd.one_shot_all_reduce(small), 500, 50)
 
     cu = ctypes.c_int()
     clk = ctypes.c_int()
@@ -219,6 +226,8 @@ def main():
             "gbs": round(algo_bytes / (rot_ms * 1e-3) / 1e9, 1), "avg_launch_us": round(rot_ms * 1e3, 2)},
         "p50_us_at_1MiB": round(p50_us, 2),
         "p99_us_at_1MiB": round(p99_us, 2),
+        "p50_us_at_1MiB_c_entry_point_only": round(p50_c_us, 2),
+        "us_per_call_at_1MiB_back_to_back": round(back_dev_ms * 1e3, 2),
         "roofline": {
             "bound": "hbm",
             "achieved": round(gbs_dev, 1),
