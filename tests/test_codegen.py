@@ -1,0 +1,50 @@
+"""What hipcc makes of the kernels, checked on the assembly it emits for gfx950 (no GPU
+needed): no packed fp32 arithmetic, no scratch memory, no scalar-cache writes, and the
+phased sum kernel small enough for two workgroups per compute unit."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from tccl_amd import build as lib_build
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+pytestmark = pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"),
+                                reason="hipcc not available")
+
+
+@pytest.fixture(scope="module", params=lib_build.SOURCES)
+def asm(request, tmp_path_factory):
+    src = os.path.join(ROOT, "tccl_amd", "csrc", request.param)
+    out = tmp_path_factory.mktemp("asm") / (request.param + ".s")
+    flags = [f for f in lib_build.HIPCC_FLAGS if f != "-fPIC"]
+    cmd = [lib_build._hipcc(), *flags, "-S", "--cuda-device-only", src, "-o", str(out)]
+    subprocess.run(cmd, check=True, capture_output=True)
+    return request.param, out.read_text()
+
+
+def test_no_packed_fp32_no_scratch_no_scalar_stores(asm):
+    name, text = asm
+    assert not re.search(r"\bv_pk_(add|mul|fma)_f32\b", text), f"{name}: packed fp32 arithmetic"
+    assert not re.search(r"\b(s_store_dword|s_buffer_store|s_dcache_wb|s_dcache_inv|s_atomic_)", text), name
+    sizes = [int(m) for m in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)]
+    assert all(s == 0 for s in sizes), f"{name}: a kernel uses scratch memory"
+    if name != "util.hip":                 # util.hip is host code only
+        assert sizes and ".wavefront_size: 64" in text
+
+
+def test_phased_kernels_fit_two_workgroups_per_cu(asm):
+    name, text = asm
+    if name != "sum.hip":
+        pytest.skip("only the sum kernels")
+    # every kernel record: name ... vgpr_count
+    records = re.findall(r"\.name:\s+(\S*sum_phased_kernel\S*)\n(?:.*\n)*?\s+\.vgpr_count:\s+(\d+)", text)
+    assert len(records) >= 32
+    for kernel, vgprs in records:
+        # 256 lanes = one wave per SIMD per workgroup; two workgroups need <= 256 VGPRs each
+        assert int(vgprs) <= 256, (kernel, vgprs)
+    w8 = [int(v) for k, v in records if "Bf16SumELi8ELi1ELb1" in k]
+    assert w8 and w8[0] <= 256
+    assert "v_cvt_pk_bf16_f32" in text and "buffer_load_dwordx4" in text and "buffer_store_dwordx4" in text
