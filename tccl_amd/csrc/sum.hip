@@ -113,11 +113,10 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
         kcount = kmax / 8 > 0 ? kmax / 8 : 1;
         wgs = (nvec + kcount * span - 1) / (kcount * span);
     } else {
-        // A bf16 input that one workgroup per compute unit can cover with full-size tiles is
+        // An input that one workgroup per compute unit can cover with full-size tiles is
         // given exactly that (measured 2-9 % better than two smaller tiles per unit at
-        // 16-32 MiB of output); anything larger runs two workgroups per unit.  fp32 inputs
-        // measured the other way round (one per unit 20 % slower) and keep two.
-        if (Sum::kElemBytes == 2 && !(cfg && cfg->grid > 0) && nvec <= (wgs / 2) * span * kmax) wgs /= 2;
+        // 16-32 MiB of output); anything larger runs two workgroups per unit.
+        if (!(cfg && cfg->grid > 0) && nvec <= (wgs / 2) * span * kmax) wgs /= 2;
         // Fewest launches that fit, then the smallest tile that covers a launch's share
         // with `wgs` workgroups, so that every launch is one full, even wave of workgroups.
         size_t launches = (nvec + wgs * span * kmax - 1) / (wgs * span * kmax);
