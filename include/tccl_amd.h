@@ -177,7 +177,7 @@ int tccl_double_tree_all_reduce_fused(void *const *bufs, void *const *outs, int 
                                       int dtype, void *stream);
 
 /* The same collective recorded once into a HIP graph and replayed with one launch, for
- * callers that repeat it on the same buffers (its 2*log2(world)+1 launches cost more than
+ * callers that repeat it on the same buffers (its 2*log2(world) launches cost more than
  * its kernels below a few MiB).  No counterpart in the reference, whose whole collective
  * is one kernel per rank.  Creating a plan allocates host and driver memory (never device
  * memory) and does not run anything; launching it is asynchronous on `stream`.  A plan

@@ -161,8 +161,8 @@ def all_reduce(tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
     raise ValueError(f"unknown all-reduce algorithm {algorithm!r}")
 
 
-# Below this many bytes per buffer the level schedule is bound by its 2*log2(W)+1 dependent
-# launches (about 37 us for W=8 whatever the size) and the one-launch kernel is used instead.
+# Below this many bytes per buffer the level schedule is bound by its 2*log2(W) dependent
+# launches (about 27 us for W=8 whatever the size) and the one-launch kernel is used instead.
 FUSED_TREE_MAX_BYTES = 8 << 20
 
 

@@ -350,7 +350,9 @@ extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs,
                 j.src[1] = c1 >= 0 ? at(c1, t) : nullptr;
                 j.src[2] = at(r, t);
                 j.dst[0] = at(r, t);
-                j.dst[1] = nullptr;
+                // the extra node's step produces the final result: it goes to that rank's
+                // output in the same pass (the result is also what its buffer keeps)
+                j.dst[1] = (h == height) ? out_at(r, t) : nullptr;
                 j.numel = len[t];
                 j.is_copy = 0;
                 batch.push_back(j);
@@ -360,9 +362,9 @@ extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs,
         if (rc != TCCL_OK) return rc;
     }
 
-    // Down-sweep: the extra node already holds the result; it only has to fill its output.
-    // Every other rank copies its parent's buffer into its own buffer and its output.
-    for (int h = height; h >= 0; --h) {
+    // Down-sweep: the extra node already holds the result (and has written its output);
+    // every other rank copies its parent's buffer into its own buffer and its output.
+    for (int h = height - 1; h >= 0; --h) {
         for (int t = 0; t < 2; ++t) {
             if (len[t] == 0) continue;
             for (int r = 0; r < world; ++r) {
@@ -370,15 +372,9 @@ extern "C" int tccl_double_tree_all_reduce(void *const *bufs, void *const *outs,
                 tccl_node_job j = {};
                 j.is_copy = 1;
                 j.numel = len[t];
-                if (h == height) {
-                    if (out_at(r, t) == nullptr) continue;
-                    j.src[0] = at(r, t);
-                    j.dst[0] = out_at(r, t);
-                } else {
-                    j.src[0] = at(nbr[t][r][0], t);
-                    j.dst[0] = at(r, t);
-                    j.dst[1] = out_at(r, t);
-                }
+                j.src[0] = at(nbr[t][r][0], t);
+                j.dst[0] = at(r, t);
+                j.dst[1] = out_at(r, t);
                 batch.push_back(j);
             }
         }
