@@ -88,7 +88,7 @@ sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_
     const size_t left = bytes > off ? bytes - off : 0;
     const uint32_t valid = static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes);
     char *const dst[1] = {out};
-    sum_tile_phased<Sum, NSRC, 1, U, KMAX, FULL>(src.p, dst, off, valid, kcount);
+    sum_tile_phased<Sum, NSRC, 1, U, KMAX, FULL, Sum::kPaceLoads>(src.p, dst, off, valid, kcount);
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
 }
 

@@ -54,8 +54,8 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
 // bf16 sums: eight fp32 accumulators per 16-byte vector.
 struct Bf16Sum {
     static constexpr int kElemBytes = 2;
-    // sixteen conversions and adds per vector pace the loads already (5-10 outstanding per
-    // lane as compiled); forcing the barrier measured the same within noise
+    // large tiles: sixteen conversions and adds per vector pace the loads already (5-10
+    // outstanding per lane as compiled); forcing the barrier measured the same within noise
     static constexpr bool kPaceLoads = false;
     float a[8];
 
@@ -94,7 +94,7 @@ struct Bf16Sum {
 // fp32 sums: four accumulators per vector, no final rounding.
 struct F32Sum {
     static constexpr int kElemBytes = 4;
-    static constexpr bool kPaceLoads = true;
+    static constexpr bool kPaceLoads = true; // large tiles: see sum_tile_phased
     float a[4];
 
     __device__ __forceinline__ void zero()
@@ -261,7 +261,7 @@ struct PhasedUnroll {
 // iterations of kPhasedBlock * U vectors.  valid is a multiple of 16 (may be 0).
 // FULL = the tile has exactly KMAX iterations: straight-line code, which lets the
 // compiler start the loads of the next iteration before the adds of this one.
-template <class Sum, int NSRC, int NDST, int U, int KMAX, bool FULL>
+template <class Sum, int NSRC, int NDST, int U, int KMAX, bool FULL, bool PACE = false>
 __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], char *const (&dst)[NDST],
                                                 size_t tile_off, uint32_t valid_bytes, int kcount)
 {
@@ -290,12 +290,13 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
                 for (int s = 0; s < NSRC; ++s) acc.add(v[u][s]);
                 r[k][u] = acc.result();
             }
-            // Keep the loads of later iterations behind this iteration's adds.  The memory
-            // system runs best with about 8-16 loads of 16 bytes outstanding per lane at
-            // two waves per SIMD; left alone, the compiler hoists as many loads as it has
-            // registers for (30+ with the four adds per vector of fp32), which measured
-            // 7 % slower.
-            if constexpr (Sum::kPaceLoads) __builtin_amdgcn_sched_barrier(0);
+            // PACE: keep the loads of later iterations behind this iteration's adds.  With
+            // 128 KiB tiles at two waves per SIMD the memory system runs best with about
+            // 8-16 loads of 16 bytes outstanding per lane; left alone, the compiler hoists
+            // as many loads as it has registers for (30+ with the four adds per vector of
+            // fp32), which measured 7 % slower there.  (With the 32 KiB tiles of the tree
+            // level kernel the barrier measured 1-5 % slower, so it is not used there.)
+            if constexpr (PACE) __builtin_amdgcn_sched_barrier(0);
         }
     }
 #pragma unroll
