@@ -431,7 +431,12 @@ def run_sweep(torch, tccl_amd, lib, device):
     # whole double-tree all-reduce, W=8 x 256 MiB
     g = make_world(tccl_amd, torch, 8, 134_217_728, torch.bfloat16, device)
     _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g), 5, 2)
-    emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20, ms=round(dev_ms, 3))
+    emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20, schedule="one launch per tree level",
+         ms=round(dev_ms, 3))
+    _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True), 5, 2)
+    emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20,
+         schedule="one persistent launch, ranks signal each other per 128 KiB chunk", ms=round(dev_ms, 3),
+         expired_waits=tccl_amd.double_tree_pipelined_timeouts(g))
     drop(g)
 
 

@@ -188,6 +188,44 @@ int tccl_double_tree_plan_create(void *const *bufs, void *const *outs, int world
 int tccl_plan_launch(tccl_plan *plan, void *stream);
 int tccl_plan_destroy(tccl_plan *plan);
 
+/* The same collective as ONE persistent launch with device-side signalling, for worlds of
+ * 2, 4 or 8: each virtual rank owns a share of the grid's workgroups, which walk the
+ * pipelining chunks of both trees and run the per-rank program the reference's kernel is
+ * designed as (triton_double_tree_allreduce.py:254-335): wait for the children's chunk,
+ * reduce it with the own chunk in place, signal the parent; wait for the parent's result,
+ * copy it into the own buffer and the output, signal the children.  Replaces the
+ * wait/send pair of triton_double_tree_allreduce.py:175-225 and the signal-pad addressing
+ * of triton_barrier.py:39-142 (a sender writes into the RECEIVER's pad, the receiver polls
+ * its own pad and resets the slot), with one slot per (tree, chunk, sender) so that a send
+ * never blocks.  Leaves memory in the same final state as tccl_double_tree_all_reduce().
+ *
+ * signal_pads: HOST array of `world` device pointers (the reference's
+ *   symm_mem.signal_pad_ptrs_dev), each to pad_bytes >= tccl_double_tree_signal_pad_bytes()
+ *   bytes, 16-byte aligned and ZERO-FILLED before the first call.  A completed call leaves
+ *   them zero-filled again.  The last word of pad 0 counts time-outs.
+ * Waits are bounded (cfg->spin_limit polls): a workgroup whose signal never comes counts a
+ *   time-out and leaves the kernel, and so does everyone who waits for it, so the launch
+ *   always ends; the buffers then hold partial results and the pads must be cleared by the
+ *   caller.  tccl_double_tree_pipelined_timeouts() reads the count (it synchronises the stream).
+ * Every workgroup of the launch must be resident at the same time: the library sizes the
+ *   grid from the occupancy HIP reports, and a device must run only ONE pipelined call at a
+ *   time (two overlapping ones can starve each other until they time out). */
+typedef struct {
+    int workgroups;      /* total workgroups (all ranks); 0 = as many as are resident at once */
+    int lag;             /* 1 + rounds the down-sweep runs behind the up-sweep; 0 = default (2) */
+    unsigned spin_limit; /* polls before a wait gives up; 0 = default (about a second) */
+    int tile_kib;        /* a workgroup works a chunk in tiles of 32 (default) or 128 KiB */
+} tccl_pipeline_cfg;
+
+size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int dtype, size_t chunk_elems);
+int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs,
+                                          void *const *signal_pads, size_t pad_bytes, int world,
+                                          size_t numel, int dtype, size_t chunk_elems,
+                                          const tccl_pipeline_cfg *cfg, void *stream);
+int tccl_double_tree_pipelined_timeouts(void *const *signal_pads, int world, size_t numel,
+                                        int dtype, size_t chunk_elems, unsigned *timeouts_out,
+                                        void *stream);
+
 /* HIP-event helpers so a host language without HIP bindings can time launches on the very
  * stream they run on.  No counterpart in the reference (it times with torch.cuda.Event,
  * triton_reduce_scatter.py:216-226). */

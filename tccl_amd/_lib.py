@@ -13,6 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtccl_amd.so")
 
 ABI_VERSION = 1
+TCCL_OK, TCCL_EINVAL, TCCL_EALIGN, TCCL_EPOW2 = 0, -1, -2, -3
 MAX_WORLD = 8
 MAX_JOBS = 8
 
@@ -39,6 +40,12 @@ class LaunchCfg(ctypes.Structure):
     """Mirror of ``tccl_launch_cfg``; any field left 0 is chosen by the library."""
     _fields_ = [("block", ctypes.c_int), ("unroll", ctypes.c_int), ("grid", ctypes.c_int),
                 ("tile_iters", ctypes.c_int), ("flags", ctypes.c_int)]
+
+
+class PipelineCfg(ctypes.Structure):
+    """Mirror of ``tccl_pipeline_cfg``; any field left 0 is chosen by the library."""
+    _fields_ = [("workgroups", ctypes.c_int), ("lag", ctypes.c_int), ("spin_limit", ctypes.c_uint),
+                ("tile_kib", ctypes.c_int)]
 
 
 class NodeJob(ctypes.Structure):
@@ -71,6 +78,10 @@ SIGNATURES = {
     "tccl_double_tree_split": (_SZ, [_SZ, _SZ]),
     "tccl_double_tree_all_reduce": (_I, [_PP, _PP, _I, _SZ, _I, _SZ, _P]),
     "tccl_double_tree_all_reduce_fused": (_I, [_PP, _PP, _I, _SZ, _I, _P]),
+    "tccl_double_tree_signal_pad_bytes": (_SZ, [_I, _SZ, _I, _SZ]),
+    "tccl_double_tree_all_reduce_pipelined": (_I, [_PP, _PP, _PP, _SZ, _I, _SZ, _I, _SZ,
+                                                   ctypes.POINTER(PipelineCfg), _P]),
+    "tccl_double_tree_pipelined_timeouts": (_I, [_PP, _I, _SZ, _I, _SZ, ctypes.POINTER(ctypes.c_uint), _P]),
     "tccl_double_tree_plan_create": (_I, [_PP, _PP, _I, _SZ, _I, _SZ, _PP]),
     "tccl_plan_launch": (_I, [_P, _P]),
     "tccl_plan_destroy": (_I, [_P]),

@@ -167,7 +167,8 @@ FUSED_TREE_MAX_BYTES = 8 << 20
 
 
 def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tensor,
-                     chunk_elems: int, fused: Optional[bool] = None) -> List[torch.Tensor]:
+                     chunk_elems: int, fused: Optional[bool] = None, pipelined: bool = False,
+                     pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> List[torch.Tensor]:
     # one allocation for all W outputs (rows are 16-byte aligned: numel is whole vectors)
     stacked = torch.empty((group.world_size,) + tuple(like.shape), dtype=like.dtype, device=like.device)
     outputs = list(stacked.unbind(0))
@@ -175,6 +176,16 @@ def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tenso
     row_bytes = like.numel() * like.element_size()
     first = int(stacked.data_ptr())
     out_ptrs = _lib.ptr_array([first + r * row_bytes for r in range(group.world_size)])
+    if pipelined:
+        need = lib.tccl_double_tree_signal_pad_bytes(group.world_size, numel, dtype, chunk_elems)
+        if need == 0:
+            raise ValueError("the pipelined double tree needs a world of 2, 4 or 8 and whole 16-byte vectors")
+        pads = group.signal_pads(need)
+        rc = lib.tccl_double_tree_all_reduce_pipelined(
+            group.ptr_array, out_ptrs, pads, group.signal_pad_bytes, group.world_size, numel, dtype, chunk_elems,
+            ctypes.byref(pipeline_cfg) if pipeline_cfg is not None else None, _stream(like.device))
+        _lib.check("tccl_double_tree_all_reduce_pipelined", rc)
+        return outputs
     if fused is None:
         fused = group.world_size <= 8 and numel * like.element_size() <= FUSED_TREE_MAX_BYTES
     if fused:
@@ -229,15 +240,37 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
 
 
 def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *,
-                                 chunk_elems: int = 0, fused: Optional[bool] = None) -> List[torch.Tensor]:
-    """One whole collective for every virtual rank of ``group``; returns the W outputs."""
+                                 chunk_elems: int = 0, fused: Optional[bool] = None, pipelined: bool = False,
+                                 pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> List[torch.Tensor]:
+    """One whole collective for every virtual rank of ``group``; returns the W outputs.
+
+    ``pipelined``: one persistent launch in which the ranks' workgroups hand chunks to each
+    other through the group's signal pads (the reference kernel's wait/reduce/send design,
+    triton_double_tree_allreduce.py:254-335) instead of one launch per tree level.  Check
+    ``double_tree_pipelined_timeouts`` afterwards when a wait may have expired."""
     like = group.tensors[0].reshape(-1)
     if numel is not None:
         like = like[:numel]
     dtype = _sum_dtype(like)
     assert like.numel() % _vec_elems(like) == 0, "The number of elements must be 128-bit aligned."
     group.pending_outputs.clear()
-    return _run_double_tree(group, like.numel(), dtype, like, chunk_elems, fused)
+    return _run_double_tree(group, like.numel(), dtype, like, chunk_elems, fused, pipelined, pipeline_cfg)
+
+
+def double_tree_pipelined_timeouts(group: SymmGroup, numel: Optional[int] = None, *, chunk_elems: int = 0) -> int:
+    """Waits of pipelined calls on ``group`` that expired since its pads were last cleared
+    (0 after correct runs).  Synchronises the current stream."""
+    like = group.tensors[0].reshape(-1)
+    if numel is not None:
+        like = like[:numel]
+    if group.signal_pad_bytes == 0:
+        return 0
+    count = ctypes.c_uint(0)
+    rc = _lib.load().tccl_double_tree_pipelined_timeouts(
+        group.signal_pads(group.signal_pad_bytes), group.world_size, like.numel(), _sum_dtype(like), chunk_elems,
+        ctypes.byref(count), _stream(like.device))
+    _lib.check("tccl_double_tree_pipelined_timeouts", rc)
+    return int(count.value)
 
 
 class DoubleTreePlan:

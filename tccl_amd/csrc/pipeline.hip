@@ -1,0 +1,401 @@
+// pipeline.hip -- the double tree as ONE persistent launch in which every virtual rank's
+// workgroups hand pipelining chunks to each other through signal flags, the way the
+// reference's per-rank kernel is designed to (triton_double_tree_allreduce.py:254-335:
+// wait for the children, reduce, signal the parent, wait for the parent, copy, signal
+// the children), with its wait/send pair (triton_double_tree_allreduce.py:175-225) and its
+// signal-pad addressing (a sender writes slot `block * world + sender` of the receiver's
+// pad; triton_barrier.py:39-142) rewritten for gfx950.
+//
+// Differences from the reference's protocol, on purpose:
+//  * one slot per (chunk, sender) instead of one per (block, sender), so a sender never has
+//    to wait for the receiver to drain the previous chunk's signal (the reference's send
+//    spins on a compare-and-swap 0 -> 1 for that); every slot has exactly one writer and
+//    one reader per call, so plain release stores and acquire loads replace the
+//    compare-and-swap loops;
+//  * the reader writes the slot back to 0 after it has seen the signal, so a pad that starts
+//    zero-filled is zero-filled again after every completed call (the property that makes the
+//    reference's barrier usable under graph replay);
+//  * every wait is bounded: a workgroup that polls `spin_limit` times without seeing its
+//    signal counts one time-out in the status word and leaves the kernel; whoever waits for
+//    that workgroup then times out the same way, so the grid always drains.
+//
+// Forward progress needs every workgroup of the launch resident at once: the grid is sized
+// from the occupancy the runtime reports for the kernel.  Two such launches that overlap in
+// time on one GPU could each hold half the slots and starve each other until the time-out,
+// so a device runs one pipelined call at a time.
+#include <mutex>
+
+#include "host.h"
+#include "vec.h"
+
+namespace tccl {
+
+constexpr int kPipeMaxWorld = TCCL_MAX_WORLD;
+constexpr uint32_t kPipeDefaultSpins = 1u << 21;
+
+struct PipeArgs {
+    char *buf[kPipeMaxWorld];
+    char *out[kPipeMaxWorld]; // entries may be null
+    uint32_t *pad[kPipeMaxWorld];
+    signed char nbr[2][kPipeMaxWorld][3]; // parent, child0, child1 (-1 = none)
+    signed char height[2][kPipeMaxWorld]; // 0 = leaf ... tree_height = the extra node on top
+    size_t half_off[2];                   // byte offset of each tree's half inside a buffer
+    size_t half_bytes[2];
+    uint32_t nchunks[2];
+    uint32_t chunk_bytes; // multiple of 16
+    uint32_t slots;       // chunk slots per tree in a pad (>= both nchunks)
+    uint32_t spin_limit;
+    int world, wgs_per_rank, lag, tree_height;
+    uint32_t *status; // time-out counter
+};
+
+// Coherence between workgroups on different XCDs (each XCD has its own L2) without flushing
+// or invalidating whole caches: every store of this kernel is a device-scope store (sc1: it
+// is written through to memory and acknowledged from there) and every load of data that a
+// peer may have rewritten during the kernel is a device-scope load (sc1: it never hits a
+// stale line of the local L2).  What is left is ordering: a wave waits until all its stores
+// have been acknowledged, the workgroup meets, then one lane raises the flag.
+__device__ __forceinline__ void send_signals(uint32_t *slot0, uint32_t *slot1)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (slot0 != nullptr) __hip_atomic_store(slot0, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (slot1 != nullptr) __hip_atomic_store(slot1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// Wait until every non-null slot has been raised, and lower it again.  One lane polls (a
+// device-scope load); the result reaches the other lanes through LDS, and the barrier keeps
+// every lane's later loads behind the poll that saw the flag.  Returns false after
+// spin_limit polls without success (counted in *status); the caller then leaves the kernel.
+__device__ __forceinline__ bool wait_signals(uint32_t *slot0, uint32_t *slot1, uint32_t spin_limit, uint32_t *status,
+                                             int *lds_ok)
+{
+    if (slot0 == nullptr && slot1 == nullptr) return true; // uniform over the workgroup
+    if (threadIdx.x == 0) {
+        bool ok = true;
+        uint32_t *const slots[2] = {slot0, slot1};
+        uint32_t polls = 0;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint32_t *s = slots[i];
+            if (s == nullptr || !ok) continue;
+            while (__hip_atomic_load(s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+                if (++polls >= spin_limit) {
+                    ok = false;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (ok) __hip_atomic_store(s, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (!ok) __hip_atomic_fetch_add(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *lds_ok = ok ? 1 : 0;
+    }
+    __syncthreads();
+    const int ok = *lds_ok;
+    __syncthreads(); // lds_ok may be rewritten by the next wait only after everyone has read it
+    return ok != 0;
+}
+
+// One chunk of a reduce step: sources -> destinations, in tiles of VECS vectors per lane
+// (256 lanes: 32 KiB for VECS = 8, 128 KiB for VECS = 32), each read and reduced into
+// registers and then written.
+template <class Sum, int VECS, int NSRC, int NDST>
+__device__ __forceinline__ void reduce_chunk(const char *const (&src)[NSRC], char *const (&dst)[NDST], size_t off,
+                                             uint32_t bytes)
+{
+    constexpr int U = VECS >= 32 ? PhasedUnroll<NSRC>::value : 2;
+    constexpr int KMAX = VECS / U;
+    constexpr uint32_t span = kPhasedBlock * U * kVecBytes;
+    constexpr uint32_t kPipeTileBytes = kPhasedBlock * VECS * kVecBytes;
+    for (uint32_t done = 0; done < bytes; done += kPipeTileBytes) {
+        const uint32_t valid = bytes - done < kPipeTileBytes ? bytes - done : kPipeTileBytes;
+        const int kcount = static_cast<int>((valid + span - 1) / span);
+        if (valid == kPipeTileBytes)
+            sum_tile_phased<Sum, NSRC, NDST, U, KMAX, true, false, kAuxLoadDevice>(src, dst, off + done, valid, KMAX);
+        else
+            sum_tile_phased<Sum, NSRC, NDST, U, KMAX, false, false, kAuxLoadDevice>(src, dst, off + done, valid, kcount);
+    }
+}
+
+template <int VECS, int NDST>
+__device__ __forceinline__ void copy_chunk(const char *src, char *const (&dst)[NDST], size_t off, uint32_t bytes)
+{
+    constexpr int U = 4;
+    constexpr int KMAX = VECS / U;
+    constexpr uint32_t span = kPhasedBlock * U * kVecBytes;
+    constexpr uint32_t kPipeTileBytes = kPhasedBlock * VECS * kVecBytes;
+    for (uint32_t done = 0; done < bytes; done += kPipeTileBytes) {
+        const uint32_t valid = bytes - done < kPipeTileBytes ? bytes - done : kPipeTileBytes;
+        copy_tile_phased<NDST, U, KMAX, kAuxLoadDevice>(src, dst, off + done, valid, static_cast<int>((valid + span - 1) / span));
+    }
+}
+
+// Up-sweep step of `rank` in tree t for chunk c: own <- 0 + child0 + child1 + own (absent
+// children skipped), in place; the extra node on top also writes its output, because its
+// sum is the final result.  Returns false on a time-out.
+template <class Sum, int VECS>
+__device__ __forceinline__ bool up_step(const PipeArgs &a, int rank, int t, uint32_t c, int *lds_ok)
+{
+    const int h = a.height[t][rank];
+    if (h == 0) return true; // a leaf's own step changes nothing anyone can see
+    const int parent = a.nbr[t][rank][0], c0 = a.nbr[t][rank][1], c1 = a.nbr[t][rank][2];
+    const uint32_t slot = (static_cast<uint32_t>(t) * a.slots + c) * a.world;
+    // children that are leaves have nothing to signal: their buffers are the inputs
+    uint32_t *w0 = (c0 >= 0 && a.height[t][c0] > 0) ? a.pad[rank] + slot + c0 : nullptr;
+    uint32_t *w1 = (c1 >= 0 && a.height[t][c1] > 0) ? a.pad[rank] + slot + c1 : nullptr;
+    if (!wait_signals(w0, w1, a.spin_limit, a.status, lds_ok)) return false;
+
+    const size_t off = a.half_off[t] + static_cast<size_t>(c) * a.chunk_bytes;
+    const size_t left = a.half_bytes[t] - static_cast<size_t>(c) * a.chunk_bytes;
+    const uint32_t bytes = left < a.chunk_bytes ? static_cast<uint32_t>(left) : a.chunk_bytes;
+    char *own = a.buf[rank];
+    const bool top = h == a.tree_height;
+    char *out = top ? a.out[rank] : nullptr;
+    if (!top) {
+        // an interior node of the perfect tree has both children
+        const char *const src[3] = {a.buf[c0], a.buf[c1], own};
+        char *const dst[1] = {own};
+        reduce_chunk<Sum, VECS, 3, 1>(src, dst, off, bytes);
+    } else {
+        // the extra node has one child (tree.py:133-136)
+        const char *const src[2] = {a.buf[c0], own};
+        if (out != nullptr) {
+            char *const dst[2] = {own, out};
+            reduce_chunk<Sum, VECS, 2, 2>(src, dst, off, bytes);
+        } else {
+            char *const dst[1] = {own};
+            reduce_chunk<Sum, VECS, 2, 1>(src, dst, off, bytes);
+        }
+    }
+    if (!top) {
+        send_signals(a.pad[parent] + slot + rank, nullptr);
+    } else {
+        // the result is final: start the down-sweep
+        send_signals(a.pad[c0] + slot + rank, nullptr);
+    }
+    return true;
+}
+
+// Down-sweep step: own, output <- parent (triton_double_tree_allreduce.py:306-326), then
+// tell the children.
+template <int VECS>
+__device__ __forceinline__ bool down_step(const PipeArgs &a, int rank, int t, uint32_t c, int *lds_ok)
+{
+    const int h = a.height[t][rank];
+    if (h == a.tree_height) return true; // the extra node already holds and has written the result
+    const int parent = a.nbr[t][rank][0], c0 = a.nbr[t][rank][1], c1 = a.nbr[t][rank][2];
+    const uint32_t slot = (static_cast<uint32_t>(t) * a.slots + c) * a.world;
+    if (!wait_signals(a.pad[rank] + slot + parent, nullptr, a.spin_limit, a.status, lds_ok)) return false;
+
+    const size_t off = a.half_off[t] + static_cast<size_t>(c) * a.chunk_bytes;
+    const size_t left = a.half_bytes[t] - static_cast<size_t>(c) * a.chunk_bytes;
+    const uint32_t bytes = left < a.chunk_bytes ? static_cast<uint32_t>(left) : a.chunk_bytes;
+    if (a.out[rank] != nullptr) {
+        char *const dst[2] = {a.buf[rank], a.out[rank]};
+        copy_chunk<VECS, 2>(a.buf[parent], dst, off, bytes);
+    } else {
+        char *const dst[1] = {a.buf[rank]};
+        copy_chunk<VECS, 1>(a.buf[parent], dst, off, bytes);
+    }
+    if (c0 >= 0 || c1 >= 0)
+        send_signals(c0 >= 0 ? a.pad[c0] + slot + rank : nullptr, c1 >= 0 ? a.pad[c1] + slot + rank : nullptr);
+    return true;
+}
+
+// Workgroup g of a rank's wgs_per_rank takes chunks g, g + wgs_per_rank, ... of both trees.
+// In round i it runs the up-sweep steps of its i-th chunk and the down-sweep steps of its
+// (i - lag)-th.  Every rank's workgroup g walks the same chunks in the same order, and a
+// step only waits for steps of the same chunk that sit at the same or an earlier place in
+// the other ranks' order (up-sweep: lower tree levels; down-sweep: the levels above, ending
+// at the extra node's up-sweep step), so with all workgroups resident nothing waits in a
+// circle.
+template <class Sum, int VECS>
+__global__ void __launch_bounds__(kPhasedBlock) tree_pipelined_kernel(PipeArgs a)
+{
+    __shared__ int lds_ok;
+    const int rank = static_cast<int>(blockIdx.x) / a.wgs_per_rank;
+    const uint32_t g = blockIdx.x % a.wgs_per_rank;
+    const uint32_t G = a.wgs_per_rank;
+    const uint32_t most = a.nchunks[0] > a.nchunks[1] ? a.nchunks[0] : a.nchunks[1];
+    if (g >= most) return;
+    const uint32_t rounds = (most - g + G - 1) / G;
+    const uint32_t lag = a.lag;
+    for (uint32_t i = 0; i < rounds + lag; ++i) {
+        if (i < rounds) {
+            const uint32_t c = g + i * G;
+            for (int t = 0; t < 2; ++t)
+                if (c < a.nchunks[t] && !up_step<Sum, VECS>(a, rank, t, c, &lds_ok)) return;
+        }
+        if (i >= lag) {
+            const uint32_t c = g + (i - lag) * G;
+            for (int t = 0; t < 2; ++t)
+                if (c < a.nchunks[t] && !down_step<VECS>(a, rank, t, c, &lds_ok)) return;
+        }
+    }
+}
+
+// Workgroups of a kernel that can be resident at once on the current device.
+template <class Sum, int VECS>
+static int resident_workgroups()
+{
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, tree_pipelined_kernel<Sum, VECS>, kPhasedBlock, 0) !=
+            hipSuccess ||
+        per_cu < 1)
+        return 0;
+    return per_cu * compute_units();
+}
+
+static int resident_workgroups(int dtype, int vecs)
+{
+    // asked once per kernel: the answer depends on the kernel's register use only
+    static std::once_flag once[4];
+    static int cached[4] = {0, 0, 0, 0};
+    const int i = (dtype == TCCL_BF16 ? 0 : 1) + (vecs == 8 ? 0 : 2);
+    std::call_once(once[i], [&] {
+        switch (i) {
+        case 0: cached[i] = resident_workgroups<Bf16Sum, 8>(); break;
+        case 1: cached[i] = resident_workgroups<F32Sum, 8>(); break;
+        case 2: cached[i] = resident_workgroups<Bf16Sum, 32>(); break;
+        default: cached[i] = resident_workgroups<F32Sum, 32>(); break;
+        }
+    });
+    return cached[i];
+}
+
+static bool pow2_small_world(int world) { return world == 2 || world == 4 || world == 8; }
+
+struct PipeGeometry {
+    size_t per_vec, split, chunk_bytes;
+    size_t half_bytes[2];
+    size_t nchunks[2];
+    size_t slots; // chunk slots per tree
+};
+
+static int pipe_geometry(int world, size_t numel, int dtype, size_t chunk_elems, PipeGeometry *g)
+{
+    const int esize = dtype_size(dtype);
+    if (esize == 0) return TCCL_EINVAL;
+    if (!pow2_small_world(world)) return (world >= 2 && (world & (world - 1)) == 0) ? TCCL_EINVAL : TCCL_EPOW2;
+    g->per_vec = kVecBytes / esize;
+    if (numel % g->per_vec != 0) return TCCL_EALIGN;
+    if (chunk_elems == 0) chunk_elems = (128u * 1024u) / esize;
+    if (chunk_elems % g->per_vec != 0) return TCCL_EALIGN;
+    g->chunk_bytes = chunk_elems * esize;
+    if (g->chunk_bytes > (static_cast<size_t>(1) << 30)) return TCCL_EINVAL;
+    g->split = tccl_double_tree_split(numel, esize);
+    g->half_bytes[0] = g->split * esize;
+    g->half_bytes[1] = (numel - g->split) * esize;
+    for (int t = 0; t < 2; ++t) g->nchunks[t] = (g->half_bytes[t] + g->chunk_bytes - 1) / g->chunk_bytes;
+    g->slots = g->nchunks[0] > g->nchunks[1] ? g->nchunks[0] : g->nchunks[1];
+    if (g->slots > 0x0FFFFFFFu) return TCCL_EINVAL;
+    return TCCL_OK;
+}
+
+} // namespace tccl
+
+using namespace tccl;
+
+extern "C" size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int dtype, size_t chunk_elems)
+{
+    PipeGeometry g;
+    if (pipe_geometry(world, numel, dtype, chunk_elems, &g) != TCCL_OK) return 0;
+    // two trees x slots x world flags, then the status word; rounded up to 16 bytes
+    const size_t words = 2 * g.slots * static_cast<size_t>(world) + 1;
+    return (words * sizeof(uint32_t) + 15) / 16 * 16;
+}
+
+extern "C" int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs, void *const *signal_pads,
+                                                     size_t pad_bytes, int world, size_t numel, int dtype,
+                                                     size_t chunk_elems, const tccl_pipeline_cfg *cfg, void *stream)
+{
+    if (bufs == nullptr || signal_pads == nullptr) return TCCL_EINVAL;
+    PipeGeometry g;
+    int rc = pipe_geometry(world, numel, dtype, chunk_elems, &g);
+    if (rc != TCCL_OK) return rc;
+    const size_t need = tccl_double_tree_signal_pad_bytes(world, numel, dtype, chunk_elems);
+    if (pad_bytes < need) return TCCL_EINVAL;
+    for (int r = 0; r < world; ++r) {
+        if (bufs[r] == nullptr || signal_pads[r] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(bufs[r]) || !aligned16(signal_pads[r]) || (outs && !aligned16(outs[r]))) return TCCL_EALIGN;
+    }
+    if (numel == 0) return TCCL_OK;
+
+    PipeArgs a = {};
+    int height = 0;
+    while ((1 << height) < world) ++height;
+    a.tree_height = height;
+    for (int r = 0; r < world; ++r) {
+        a.buf[r] = static_cast<char *>(bufs[r]);
+        a.out[r] = outs ? static_cast<char *>(outs[r]) : nullptr;
+        a.pad[r] = static_cast<uint32_t *>(signal_pads[r]);
+        int six[6];
+        rc = tccl_double_tree_indices(world, r, six);
+        if (rc != TCCL_OK) return rc;
+        for (int t = 0; t < 2; ++t) {
+            for (int k = 0; k < 3; ++k) a.nbr[t][r][k] = static_cast<signed char>(six[3 * t + k]);
+            const int ra = (t == 0) ? r : (r + 1) % world; // the rank's label in tree a's numbering
+            a.height[t][r] = static_cast<signed char>(ra == 0 ? height : __builtin_ctz(ra));
+        }
+    }
+    const int esize = dtype_size(dtype);
+    a.half_off[0] = 0;
+    a.half_off[1] = g.split * esize;
+    for (int t = 0; t < 2; ++t) {
+        a.half_bytes[t] = g.half_bytes[t];
+        a.nchunks[t] = static_cast<uint32_t>(g.nchunks[t]);
+    }
+    a.chunk_bytes = static_cast<uint32_t>(g.chunk_bytes);
+    a.slots = static_cast<uint32_t>(g.slots);
+    a.world = world;
+    a.status = a.pad[0] + 2 * g.slots * world;
+    a.spin_limit = (cfg && cfg->spin_limit > 0) ? cfg->spin_limit : kPipeDefaultSpins;
+    a.lag = (cfg && cfg->lag > 0) ? cfg->lag - 1 : 1; // cfg->lag is 1-based so that 0 means "default"
+    if (a.lag > 64) a.lag = 64;
+
+    // Every workgroup must be resident: the grid never exceeds what the runtime says fits.
+    const int vecs = (cfg && cfg->tile_kib == 128) ? 32 : 8;
+    const int resident = resident_workgroups(dtype, vecs);
+    if (resident < world) return hip_code(hipErrorLaunchOutOfResources);
+    int wgs = (cfg && cfg->workgroups > 0) ? cfg->workgroups : resident;
+    if (wgs > resident) wgs = resident;
+    int per_rank = wgs / world;
+    if (per_rank < 1) per_rank = 1;
+    if (static_cast<size_t>(per_rank) > g.slots) per_rank = static_cast<int>(g.slots);
+    a.wgs_per_rank = per_rank;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid(static_cast<unsigned>(per_rank * world));
+    if (dtype == TCCL_BF16) {
+        if (vecs == 8)
+            hipLaunchKernelGGL((tree_pipelined_kernel<Bf16Sum, 8>), grid, dim3(kPhasedBlock), 0, s, a);
+        else
+            hipLaunchKernelGGL((tree_pipelined_kernel<Bf16Sum, 32>), grid, dim3(kPhasedBlock), 0, s, a);
+    } else {
+        if (vecs == 8)
+            hipLaunchKernelGGL((tree_pipelined_kernel<F32Sum, 8>), grid, dim3(kPhasedBlock), 0, s, a);
+        else
+            hipLaunchKernelGGL((tree_pipelined_kernel<F32Sum, 32>), grid, dim3(kPhasedBlock), 0, s, a);
+    }
+    return hip_code(hipGetLastError());
+}
+
+extern "C" int tccl_double_tree_pipelined_timeouts(void *const *signal_pads, int world, size_t numel, int dtype,
+                                                   size_t chunk_elems, unsigned *timeouts_out, void *stream)
+{
+    if (signal_pads == nullptr || signal_pads[0] == nullptr || timeouts_out == nullptr) return TCCL_EINVAL;
+    PipeGeometry g;
+    const int rc = pipe_geometry(world, numel, dtype, chunk_elems, &g);
+    if (rc != TCCL_OK) return rc;
+    const uint32_t *status = static_cast<const uint32_t *>(signal_pads[0]) + 2 * g.slots * world;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint32_t v = 0;
+    hipError_t e = hipMemcpyAsync(&v, status, sizeof(v), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_code(e);
+    *timeouts_out = v;
+    return TCCL_OK;
+}

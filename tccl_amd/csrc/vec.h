@@ -241,6 +241,7 @@ constexpr int kPhasedVecs = 32;   // result vectors a lane holds before it write
 constexpr int kAuxLoadStream = 2;   // cache policy of the loads: nt (stream through L2)
 constexpr int kAuxStoreStream = 16; // cache policy of a tile's result stores: sc1 (write through to memory)
 constexpr int kAuxStoreNt = 2;      // cache policy of the stores of streaming copies: nt
+constexpr int kAuxLoadDevice = 18;  // sc1 nt: device-scope loads, coherent with sc1 stores of other XCDs
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const char *tile_start, uint32_t valid_bytes)
 {
@@ -261,7 +262,8 @@ struct PhasedUnroll {
 // iterations of kPhasedBlock * U vectors.  valid is a multiple of 16 (may be 0).
 // FULL = the tile has exactly KMAX iterations: straight-line code, which lets the
 // compiler start the loads of the next iteration before the adds of this one.
-template <class Sum, int NSRC, int NDST, int U, int KMAX, bool FULL, bool PACE = false>
+// LAUX = cache policy of the loads.
+template <class Sum, int NSRC, int NDST, int U, int KMAX, bool FULL, bool PACE = false, int LAUX = kAuxLoadStream>
 __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], char *const (&dst)[NDST],
                                                 size_t tile_off, uint32_t valid_bytes, int kcount)
 {
@@ -281,7 +283,7 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
 #pragma unroll
                 for (int s = 0; s < NSRC; ++s)
                     v[u][s] = __builtin_amdgcn_raw_buffer_load_b128(
-                        rs[s], k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxLoadStream);
+                        rs[s], k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, LAUX);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 Sum acc;
@@ -315,7 +317,7 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
 }
 
 // Same walk for a plain copy of one source into NDST destinations.
-template <int NDST, int U, int KMAX>
+template <int NDST, int U, int KMAX, int LAUX = kAuxLoadStream>
 __device__ __forceinline__ void copy_tile_phased(const char *src, char *const (&dst)[NDST], size_t tile_off,
                                                  uint32_t valid_bytes, int kcount)
 {
@@ -329,7 +331,7 @@ __device__ __forceinline__ void copy_tile_phased(const char *src, char *const (&
 #pragma unroll
             for (int u = 0; u < U; ++u)
                 r[k][u] = __builtin_amdgcn_raw_buffer_load_b128(
-                    rs, k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxLoadStream);
+                    rs, k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, LAUX);
         }
     }
 #pragma unroll

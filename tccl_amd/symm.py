@@ -6,8 +6,10 @@ The reference allocates one peer-mappable buffer per process with
 obtains the table of all W buffer addresses with ``_SymmetricMemory.rendezvous(tensor)``
 (:82), whose handle carries ``buffer_ptrs_dev``, ``rank`` and ``world_size`` (:86-91).
 Here one process owns all W buffers; ``rendezvous`` finds the group a tensor belongs to in
-a process-local registry keyed by the address of the tensor's storage.  Signal pads do not
-exist: ordering between virtual ranks is the order of work on the HIP stream.
+a process-local registry keyed by the address of the tensor's storage.  Ordering between
+virtual ranks is the order of work on the HIP stream; signal pads (``signal_pad_ptrs_dev``,
+:87) exist only for the one kernel that signals on the device, the pipelined double tree,
+and are allocated when it is first used.
 """
 from __future__ import annotations
 
@@ -58,6 +60,29 @@ class SymmGroup:
         # double-tree bookkeeping: outputs produced by the collective that is in progress,
         # waiting to be picked up by the ranks that have not called yet
         self.pending_outputs: Dict[int, torch.Tensor] = {}
+        self._signal_pads: List[torch.Tensor] = []
+        self._signal_pad_array: Optional[ctypes.Array] = None
+
+    def signal_pads(self, nbytes: int) -> ctypes.Array:
+        """Host array of W device addresses of zero-filled signal pads of at least ``nbytes``
+        each, one allocation per virtual rank (the reference's per-rank signal pad).  The
+        pads are created on first use and replaced by larger ones when needed; the kernels
+        that use them leave them zero-filled."""
+        if not self._signal_pads or self._signal_pads[0].numel() < nbytes:
+            device = self.tensors[0].device
+            self._signal_pads = [torch.zeros(nbytes, dtype=torch.uint8, device=device)
+                                 for _ in range(self.world_size)]
+            self._signal_pad_array = _lib.ptr_array([int(p.data_ptr()) for p in self._signal_pads])
+        return self._signal_pad_array
+
+    def clear_signal_pads(self) -> None:
+        """Zero the pads again (needed only after a call that reported time-outs)."""
+        for p in self._signal_pads:
+            p.zero_()
+
+    @property
+    def signal_pad_bytes(self) -> int:
+        return self._signal_pads[0].numel() if self._signal_pads else 0
 
     def tensor(self, rank: int) -> torch.Tensor:
         return self.tensors[rank]

@@ -101,7 +101,7 @@ def test_product_does_not_import_the_oracle():
 
 
 def test_struct_layouts_match_the_header(tmp_path):
-    """sizeof/offsetof of the two structs that cross the ABI, as gcc sees the header, against
+    """sizeof/offsetof of the structs that cross the ABI, as gcc sees the header, against
     the ctypes mirrors."""
     import shutil
     import subprocess
@@ -116,6 +116,9 @@ def test_struct_layouts_match_the_header(tmp_path):
         '         offsetof(tccl_launch_cfg, tile_iters), offsetof(tccl_launch_cfg, flags));\n'
         '  printf("%zu %zu %zu %zu %zu\\n", sizeof(tccl_node_job), offsetof(tccl_node_job, src),\n'
         '         offsetof(tccl_node_job, dst), offsetof(tccl_node_job, numel), offsetof(tccl_node_job, is_copy));\n'
+        '  printf("%zu %zu %zu %zu %zu\\n", sizeof(tccl_pipeline_cfg), offsetof(tccl_pipeline_cfg, workgroups),\n'
+        '         offsetof(tccl_pipeline_cfg, lag), offsetof(tccl_pipeline_cfg, spin_limit),\n'
+        '         offsetof(tccl_pipeline_cfg, tile_kib));\n'
         '  printf("%d %d %d %d %d %d\\n", TCCL_ABI_VERSION, TCCL_MAX_WORLD, TCCL_MAX_JOBS, TCCL_BF16, TCCL_F32,\n'
         '         TCCL_CFG_PHASED);\n'
         '  return 0;\n}\n')
@@ -124,11 +127,14 @@ def test_struct_layouts_match_the_header(tmp_path):
     lines = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
     cfg = [int(x) for x in lines[0].split()]
     job = [int(x) for x in lines[1].split()]
-    consts = [int(x) for x in lines[2].split()]
+    pipe = [int(x) for x in lines[2].split()]
+    consts = [int(x) for x in lines[3].split()]
     C = _lib.LaunchCfg
     assert cfg == [ctypes.sizeof(C), C.block.offset, C.unroll.offset, C.grid.offset, C.tile_iters.offset,
                    C.flags.offset]
     J = _lib.NodeJob
     assert job == [ctypes.sizeof(J), J.src.offset, J.dst.offset, J.numel.offset, J.is_copy.offset]
+    P = _lib.PipelineCfg
+    assert pipe == [ctypes.sizeof(P), P.workgroups.offset, P.lag.offset, P.spin_limit.offset, P.tile_kib.offset]
     assert consts == [_lib.ABI_VERSION, _lib.MAX_WORLD, _lib.MAX_JOBS, _lib.TCCL_BF16, _lib.TCCL_F32,
                       _lib.CFG_PHASED]

@@ -48,3 +48,21 @@ def test_phased_kernels_fit_two_workgroups_per_cu(asm):
     w8 = [int(v) for k, v in records if "Bf16SumELi8ELi1ELb1" in k]
     assert w8 and w8[0] <= 256
     assert "v_cvt_pk_bf16_f32" in text and "buffer_load_dwordx4" in text and "buffer_store_dwordx4" in text
+
+
+def test_pipelined_kernel_uses_device_scope_accesses_and_no_cache_flushes(asm):
+    """The pipelined double tree keeps its workgroups coherent across the XCDs' L2 caches with
+    device-scope (sc1) loads and stores alone; a whole-cache write-back or invalidate per
+    signal would cost more than the chunk it guards."""
+    name, text = asm
+    if name != "pipeline.hip":
+        pytest.skip("only the pipelined kernel")
+    loads = re.findall(r"buffer_load_dwordx4[^\n]*", text)
+    stores = re.findall(r"buffer_store_dwordx4[^\n]*", text)
+    assert loads and stores
+    assert all(re.search(r"\bsc1\b", line) for line in loads), "a data load is not device-scope"
+    assert all(re.search(r"\bsc1\b", line) for line in stores), "a data store is not device-scope"
+    assert "buffer_wbl2" not in text and "buffer_inv" not in text
+    flags = re.findall(r"global_(?:load|store)_dword [^\n]*", text)
+    assert flags and all(re.search(r"\bsc1\b", line) for line in flags), "a flag access is not device-scope"
+    assert "s_sleep" in text and "global_atomic_add" in text

@@ -1,0 +1,207 @@
+"""GPU parity of the pipelined double tree (one persistent launch, virtual ranks signalling
+each other per chunk) against the CPU oracle and against the level schedule, through the C
+ABI.  Bit-exact.  Every case also checks that no wait expired and that the signal pads are
+zero-filled again afterwards."""
+import ctypes
+import gc
+
+import pytest
+import torch
+
+import tccl_amd
+from tccl_amd import _lib
+from helpers import assert_bit_equal, from_np_bits, np_bits, seeded_randn, seeded_uniform
+from oracle import torch_ref
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+# A wait that expires in the tests should do so quickly: 2^18 polls are some tenths of a second.
+SPINS = 1 << 18
+
+
+@pytest.fixture(autouse=True)
+def _gpu_hygiene():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    tccl_amd.load_library()
+    groups = []
+    yield groups
+    torch.cuda.synchronize()
+    for g in groups:
+        tccl_amd.unregister(g)
+    groups.clear()
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def upload(groups, bufs):
+    g = tccl_amd.empty_world(len(bufs), bufs[0].shape, bufs[0].dtype, DEV)
+    for r, b in enumerate(bufs):
+        g.tensor(r).copy_(b)
+    groups.append(g)
+    return g
+
+
+def cfg(workgroups=0, lag=0, spin_limit=SPINS, tile_kib=0):
+    return _lib.PipelineCfg(workgroups, lag, spin_limit, tile_kib)
+
+
+def pads_are_zero(group):
+    return all(int(p.count_nonzero().item()) == 0 for p in group._signal_pads)   # noqa: SLF001
+
+
+def run_and_check(group, want, what, **kw):
+    print(f"pipelined: {what} {kw}", flush=True)
+    outs = tccl_amd.double_tree_all_reduce_world(group, pipelined=True, **kw)
+    chunk = kw.get("chunk_elems", 0)
+    assert tccl_amd.double_tree_pipelined_timeouts(group, chunk_elems=chunk) == 0, f"{what}: a wait expired"
+    for r in range(group.world_size):
+        assert_bit_equal(outs[r], want, f"{what}: output {r}")
+        assert_bit_equal(group.tensor(r), want, f"{what}: buffer {r}")
+    assert pads_are_zero(group), f"{what}: signal pads not reset"
+    return outs
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+@pytest.mark.parametrize("tile_kib", [32, 128])
+@pytest.mark.parametrize("numel,chunk_elems", [
+    (8, 0),                         # one vector: tree b only
+    (16, 8),                        # one vector per tree, one-vector chunks
+    (8 * 12_345, 0),                # one ragged chunk per tree
+    (8 * 12_345, 512),              # hundreds of small chunks, last one ragged
+    (65_536 * 6 + 8 * 77, 0),       # whole 128 KiB chunks plus a ragged one
+    (8 * 1_000_003, 65_536 * 3),    # chunks larger than a tile
+])
+def test_pipelined_matches_oracle_and_schedule(world, maker, tile_kib, numel, chunk_elems, _gpu_hygiene, c_oracle):
+    bufs = maker(world, numel, seed_base=900)
+    want = torch_ref.double_tree_all_reduce(bufs)[0]
+    if maker is seeded_randn:
+        _, outs = c_oracle.double_tree_all_reduce_bf16([np_bits(b) for b in bufs])
+        assert_bit_equal(from_np_bits(outs[0]), want, "oracles agree")
+    g = upload(_gpu_hygiene, bufs)
+    got = run_and_check(g, want, f"W={world} n={numel} chunk={chunk_elems} tile={tile_kib}",
+                        chunk_elems=chunk_elems, pipeline_cfg=cfg(tile_kib=tile_kib))
+    g2 = upload(_gpu_hygiene, bufs)
+    levels = tccl_amd.double_tree_all_reduce_world(g2, fused=False, chunk_elems=chunk_elems)
+    for r in range(world):
+        assert_bit_equal(levels[r], got[r], f"schedule vs pipelined, output {r}")
+
+
+@pytest.mark.parametrize("tile_kib", [32, 128])
+@pytest.mark.parametrize("workgroups,lag", [(8, 1), (8, 3), (16, 1), (64, 2), (256, 1), (256, 5), (0, 1), (0, 2), (0, 4)])
+def test_pipelined_grid_and_lag(workgroups, lag, tile_kib, _gpu_hygiene):
+    """Any grid from one workgroup per rank upwards and any distance between the sweeps gives
+    the same bits."""
+    world, numel = 8, 65_536 * 40 + 4_096
+    bufs = seeded_randn(world, numel, seed_base=910)
+    want = torch_ref.double_tree_all_reduce(bufs)[0]
+    g = upload(_gpu_hygiene, bufs)
+    run_and_check(g, want, f"wgs={workgroups} lag={lag} tile={tile_kib}",
+                  pipeline_cfg=cfg(workgroups, lag, tile_kib=tile_kib))
+
+
+def test_pipelined_repeats_on_the_same_pads(_gpu_hygiene):
+    """The pads reset themselves: back-to-back collectives on one group, no clearing between."""
+    world, numel = 8, 65_536 * 9
+    g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    for round_ in range(4):
+        bufs = seeded_randn(world, numel, seed_base=920 + 10 * round_)
+        for r, b in enumerate(bufs):
+            g.tensor(r).copy_(b)
+        want = torch_ref.double_tree_all_reduce(bufs)[0]
+        run_and_check(g, want, f"round {round_}", pipeline_cfg=cfg())
+
+
+def test_pipelined_fill_rank(_gpu_hygiene):
+    """The reference's self-test: every rank fills its buffer with its rank; all outputs are
+    W(W-1)/2 (triton_one_shot_all_reduce_no_128.py:116-127)."""
+    world = 8
+    g = upload(_gpu_hygiene, [torch.full((65_536 * 4,), float(r), dtype=torch.bfloat16) for r in range(world)])
+    outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg())
+    assert tccl_amd.double_tree_pipelined_timeouts(g) == 0
+    for r in range(world):
+        assert outs[r].eq(28).all().item()
+
+
+def test_pipelined_without_outputs_through_c_abi(_gpu_hygiene):
+    """outs = NULL: only the ranks' buffers receive the result."""
+    world, numel = 4, 65_536 * 3 + 64
+    bufs = seeded_randn(world, numel, seed_base=930)
+    want = torch_ref.double_tree_all_reduce(bufs)[0]
+    g = upload(_gpu_hygiene, bufs)
+    lib = tccl_amd.load_library()
+    need = lib.tccl_double_tree_signal_pad_bytes(world, numel, _lib.TCCL_BF16, 0)
+    pads = g.signal_pads(need)
+    c = cfg()
+    s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.tccl_double_tree_all_reduce_pipelined(g.ptr_array, None, pads, g.signal_pad_bytes, world, numel,
+                                                   _lib.TCCL_BF16, 0, ctypes.byref(c), s)
+    assert rc == 0
+    assert tccl_amd.double_tree_pipelined_timeouts(g) == 0
+    for r in range(world):
+        assert_bit_equal(g.tensor(r), want, f"buffer {r}")
+
+
+def test_pipelined_full_size_properties(_gpu_hygiene):
+    """The full benchmark shape (8 x 256 MiB bf16, 128 KiB chunks): integer-valued inputs whose
+    sum is exact in every order, so the expected result is known without a CPU pass."""
+    world, numel = 8, 134_217_728
+    g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    total = torch.zeros(numel, dtype=torch.float32, device=DEV)
+    for r in range(world):
+        vals = torch.randint(-8, 9, (numel,), generator=gen, device=DEV, dtype=torch.int32).to(torch.bfloat16)
+        g.tensor(r).copy_(vals)
+        total += vals.float()
+    want = total.to(torch.bfloat16)       # |sum| <= 64: exact in bf16 at every node
+    del total
+    outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1 << 20))
+    assert tccl_amd.double_tree_pipelined_timeouts(g) == 0
+    for r in range(world):
+        assert torch.equal(outs[r], want), f"output {r}"
+        assert torch.equal(g.tensor(r), want), f"buffer {r}"
+    assert pads_are_zero(g)
+
+
+def test_pipelined_expired_waits_drain_and_recover(_gpu_hygiene):
+    """Failure handling, forced from the host: with a spin limit of one poll, waits expire (a
+    parent polls before its children can have finished a chunk).  The launch must still end,
+    report the time-outs, and the same group must work again once its pads are cleared."""
+    world, numel = 8, 65_536 * 64
+    bufs = seeded_randn(world, numel, seed_base=940)
+    want = torch_ref.double_tree_all_reduce(bufs)[0]
+    g = upload(_gpu_hygiene, bufs)
+    print("pipelined: spin limit 1", flush=True)
+    tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1))
+    torch.cuda.synchronize()                         # the grid drained
+    expired = tccl_amd.double_tree_pipelined_timeouts(g)
+    if expired == 0:                                 # every signal happened to be there already
+        for r in range(world):
+            assert_bit_equal(g.tensor(r), want, f"buffer {r}")
+        return
+    g.clear_signal_pads()
+    for r, b in enumerate(bufs):
+        g.tensor(r).copy_(b)
+    run_and_check(g, want, "after clearing the pads", pipeline_cfg=cfg())
+
+
+def test_pipelined_argument_checks(_gpu_hygiene):
+    lib = tccl_amd.load_library()
+    g = tccl_amd.empty_world(16, 64, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    with pytest.raises(ValueError):
+        tccl_amd.double_tree_all_reduce_world(g, pipelined=True)          # worlds of 2, 4, 8 only
+    g8 = tccl_amd.empty_world(8, 64, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g8)
+    need = lib.tccl_double_tree_signal_pad_bytes(8, 64, _lib.TCCL_BF16, 0)
+    pads = g8.signal_pads(need)
+    call = lib.tccl_double_tree_all_reduce_pipelined
+    assert call(g8.ptr_array, None, pads, need - 16, 8, 64, _lib.TCCL_BF16, 0, None, None) == _lib.TCCL_EINVAL
+    assert call(g8.ptr_array, None, None, need, 8, 64, _lib.TCCL_BF16, 0, None, None) == _lib.TCCL_EINVAL
+    assert call(g8.ptr_array, None, pads, need, 8, 60, _lib.TCCL_BF16, 0, None, None) == _lib.TCCL_EALIGN
+    assert call(g8.ptr_array, None, pads, need, 8, 64, _lib.TCCL_BF16, 12, None, None) == _lib.TCCL_EALIGN
+    assert call(g8.ptr_array, None, pads, need, 3, 64, _lib.TCCL_BF16, 0, None, None) == _lib.TCCL_EPOW2
+    assert call(g8.ptr_array, None, pads, need, 8, 0, _lib.TCCL_BF16, 0, None, None) == 0
