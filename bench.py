@@ -41,7 +41,9 @@ def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
-    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=150,
+                   help="untimed steps first; 150 (13 ms) because launches 30-100 after idle run 1-2 %% slower "
+                        "than the steady state while the clocks settle")
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     p.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU work budget for the baseline leg")
     p.add_argument("--no-other-ops", action="store_true",
@@ -351,6 +353,19 @@ def other_ops(torch, tccl_amd, lib, device):
     _, ms = time_steps(torch, lib, level, 32, 8)
     out["tree_copy_step_2_destinations_128MiB_gbs"] = round(3 * half * 2 / (ms * 1e-3) / 1e9, 1)
     del bufs
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    # whole double-tree all-reduce, W=8 x 256 MiB in 128 KiB chunks (4 GiB touched per call): the level
+    # schedule (one launch per tree level) and the pipelined single launch (ranks signal each other per chunk)
+    g = make_world(tccl_amd, torch, 8, 134_217_728, torch.bfloat16, device)
+    _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g), 5, 2)
+    out["double_tree_w8_256MiB_level_schedule_ms"] = round(ms, 3)
+    _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True), 5, 2)
+    out["double_tree_w8_256MiB_pipelined_ms"] = round(ms, 3)
+    out["double_tree_pipelined_expired_waits"] = tccl_amd.double_tree_pipelined_timeouts(g)
+    tccl_amd.unregister(g)
+    del g
     gc.collect()
     torch.cuda.empty_cache()
     return out

@@ -211,8 +211,9 @@ int tccl_plan_destroy(tccl_plan *plan);
  *   grid from the occupancy HIP reports, and a device must run only ONE pipelined call at a
  *   time (two overlapping ones can starve each other until they time out). */
 typedef struct {
-    int workgroups;      /* total workgroups (all ranks); 0 = as many as are resident at once */
-    int lag;             /* 1 + rounds the down-sweep runs behind the up-sweep; 0 = default (2) */
+    int workgroups;      /* total workgroups (all ranks); 0 = as many as are safely resident at once
+                            (also the upper limit) */
+    int lag;             /* 1 + rounds the down-sweep runs behind the up-sweep; 0 = default (1: none) */
     unsigned spin_limit; /* polls before a wait gives up; 0 = default (about a second) */
     int tile_kib;        /* a workgroup works a chunk in tiles of 32 (default) or 128 KiB */
 } tccl_pipeline_cfg;

@@ -246,24 +246,42 @@ static int resident_workgroups()
             hipSuccess ||
         per_cu < 1)
         return 0;
+    // Never count on a compute unit's last wave slots: a grid sized to all eight waves per
+    // SIMD that the occupancy query reports did not become resident as a whole on MI355X
+    // (its waits expired), six per compute unit and fewer always did.
+    if (per_cu > 6) per_cu = 6;
     return per_cu * compute_units();
 }
 
-static int resident_workgroups(int dtype, int vecs)
+template <class Sum, int VECS>
+static int launch_pipelined(const PipeArgs &a, int wgs_wanted, int world, size_t slots, hipStream_t s)
 {
     // asked once per kernel: the answer depends on the kernel's register use only
-    static std::once_flag once[4];
-    static int cached[4] = {0, 0, 0, 0};
-    const int i = (dtype == TCCL_BF16 ? 0 : 1) + (vecs == 8 ? 0 : 2);
-    std::call_once(once[i], [&] {
-        switch (i) {
-        case 0: cached[i] = resident_workgroups<Bf16Sum, 8>(); break;
-        case 1: cached[i] = resident_workgroups<F32Sum, 8>(); break;
-        case 2: cached[i] = resident_workgroups<Bf16Sum, 32>(); break;
-        default: cached[i] = resident_workgroups<F32Sum, 32>(); break;
-        }
-    });
-    return cached[i];
+    static std::once_flag once;
+    static int resident = 0;
+    std::call_once(once, [] { resident = resident_workgroups<Sum, VECS>(); });
+    // Every workgroup must be resident: the grid never exceeds what the runtime says fits.
+    if (resident < world) return hip_code(hipErrorLaunchOutOfResources);
+    int wgs = wgs_wanted > 0 ? wgs_wanted : resident;
+    if (wgs > resident) wgs = resident;
+    int per_rank = wgs / world;
+    if (per_rank < 1) per_rank = 1;
+    if (static_cast<size_t>(per_rank) > slots) per_rank = static_cast<int>(slots);
+    PipeArgs args = a;
+    args.wgs_per_rank = per_rank;
+    hipLaunchKernelGGL((tree_pipelined_kernel<Sum, VECS>), dim3(static_cast<unsigned>(per_rank * world)),
+                       dim3(kPhasedBlock), 0, s, args);
+    return hip_code(hipGetLastError());
+}
+
+template <class Sum>
+static int launch_pipelined_tile(const PipeArgs &a, int tile_kib, int wgs_wanted, int world, size_t slots,
+                                 hipStream_t s)
+{
+    switch (tile_kib) {
+    case 128: return launch_pipelined<Sum, 32>(a, wgs_wanted, world, slots, s);
+    default: return launch_pipelined<Sum, 8>(a, wgs_wanted, world, slots, s);
+    }
 }
 
 static bool pow2_small_world(int world) { return world == 2 || world == 4 || world == 8; }
@@ -353,34 +371,14 @@ extern "C" int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *co
     a.world = world;
     a.status = a.pad[0] + 2 * g.slots * world;
     a.spin_limit = (cfg && cfg->spin_limit > 0) ? cfg->spin_limit : kPipeDefaultSpins;
-    a.lag = (cfg && cfg->lag > 0) ? cfg->lag - 1 : 1; // cfg->lag is 1-based so that 0 means "default"
+    a.lag = (cfg && cfg->lag > 0) ? cfg->lag - 1 : 0; // cfg->lag is 1-based so that 0 means "default"
     if (a.lag > 64) a.lag = 64;
 
-    // Every workgroup must be resident: the grid never exceeds what the runtime says fits.
-    const int vecs = (cfg && cfg->tile_kib == 128) ? 32 : 8;
-    const int resident = resident_workgroups(dtype, vecs);
-    if (resident < world) return hip_code(hipErrorLaunchOutOfResources);
-    int wgs = (cfg && cfg->workgroups > 0) ? cfg->workgroups : resident;
-    if (wgs > resident) wgs = resident;
-    int per_rank = wgs / world;
-    if (per_rank < 1) per_rank = 1;
-    if (static_cast<size_t>(per_rank) > g.slots) per_rank = static_cast<int>(g.slots);
-    a.wgs_per_rank = per_rank;
-
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const dim3 grid(static_cast<unsigned>(per_rank * world));
-    if (dtype == TCCL_BF16) {
-        if (vecs == 8)
-            hipLaunchKernelGGL((tree_pipelined_kernel<Bf16Sum, 8>), grid, dim3(kPhasedBlock), 0, s, a);
-        else
-            hipLaunchKernelGGL((tree_pipelined_kernel<Bf16Sum, 32>), grid, dim3(kPhasedBlock), 0, s, a);
-    } else {
-        if (vecs == 8)
-            hipLaunchKernelGGL((tree_pipelined_kernel<F32Sum, 8>), grid, dim3(kPhasedBlock), 0, s, a);
-        else
-            hipLaunchKernelGGL((tree_pipelined_kernel<F32Sum, 32>), grid, dim3(kPhasedBlock), 0, s, a);
-    }
-    return hip_code(hipGetLastError());
+    const int tile_kib = cfg ? cfg->tile_kib : 0;
+    const int wgs = cfg ? cfg->workgroups : 0;
+    return dtype == TCCL_BF16 ? launch_pipelined_tile<Bf16Sum>(a, tile_kib, wgs, world, g.slots, s)
+                              : launch_pipelined_tile<F32Sum>(a, tile_kib, wgs, world, g.slots, s);
 }
 
 extern "C" int tccl_double_tree_pipelined_timeouts(void *const *signal_pads, int world, size_t numel, int dtype,
