@@ -363,7 +363,17 @@ def other_ops(torch, tccl_amd, lib, device):
     out["double_tree_w8_256MiB_level_schedule_ms"] = round(ms, 3)
     _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True), 5, 2)
     out["double_tree_w8_256MiB_pipelined_ms"] = round(ms, 3)
-    out["double_tree_pipelined_expired_waits"] = tccl_amd.double_tree_pipelined_timeouts(g)
+    out["double_tree_pipelined_expired_waits"] = tccl_amd.signal_pad_timeouts(g)
+    tccl_amd.unregister(g)
+    del g
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    # all W ranks' all-reduce in place in one launch (two-shot with the blockwise barrier), 8 x 64 MiB
+    g = make_world(tccl_amd, torch, 8, 33_554_432, torch.bfloat16, device)
+    _, ms = time_steps(torch, lib, lambda: tccl_amd.two_shot_all_reduce_world(g, with_outputs=False), 20, 5)
+    out["two_shot_in_place_all_ranks_w8_64MiB_us"] = round(ms * 1e3, 1)
+    out["two_shot_expired_waits"] = tccl_amd.signal_pad_timeouts(g)
     tccl_amd.unregister(g)
     del g
     gc.collect()
@@ -451,7 +461,7 @@ def run_sweep(torch, tccl_amd, lib, device):
     _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True), 5, 2)
     emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20,
          schedule="one persistent launch, ranks signal each other per 128 KiB chunk", ms=round(dev_ms, 3),
-         expired_waits=tccl_amd.double_tree_pipelined_timeouts(g))
+         expired_waits=tccl_amd.signal_pad_timeouts(g))
     drop(g)
 
 

@@ -202,11 +202,11 @@ int tccl_plan_destroy(tccl_plan *plan);
  * signal_pads: HOST array of `world` device pointers (the reference's
  *   symm_mem.signal_pad_ptrs_dev), each to pad_bytes >= tccl_double_tree_signal_pad_bytes()
  *   bytes, 16-byte aligned and ZERO-FILLED before the first call.  A completed call leaves
- *   them zero-filled again.  The last word of pad 0 counts time-outs.
+ *   them zero-filled again.  The last 32-bit word of pad 0 (at pad_bytes - 4) counts time-outs.
  * Waits are bounded (cfg->spin_limit polls): a workgroup whose signal never comes counts a
  *   time-out and leaves the kernel, and so does everyone who waits for it, so the launch
  *   always ends; the buffers then hold partial results and the pads must be cleared by the
- *   caller.  tccl_double_tree_pipelined_timeouts() reads the count (it synchronises the stream).
+ *   caller.  tccl_signal_pad_timeouts() reads the count (it synchronises the stream).
  * Every workgroup of the launch must be resident at the same time: the library sizes the
  *   grid from the occupancy HIP reports, and a device must run only ONE pipelined call at a
  *   time (two overlapping ones can starve each other until they time out). */
@@ -223,9 +223,26 @@ int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs,
                                           void *const *signal_pads, size_t pad_bytes, int world,
                                           size_t numel, int dtype, size_t chunk_elems,
                                           const tccl_pipeline_cfg *cfg, void *stream);
-int tccl_double_tree_pipelined_timeouts(void *const *signal_pads, int world, size_t numel,
-                                        int dtype, size_t chunk_elems, unsigned *timeouts_out,
-                                        void *stream);
+int tccl_signal_pad_timeouts(const void *pad0, size_t pad_bytes, unsigned *timeouts_out,
+                             void *stream);
+
+/* Two-shot all-reduce for all virtual ranks in ONE launch, in place: afterwards every
+ * bufs[r] (and every outs[r], if given) holds sum_i bufs[i] -- each element the fp32 sum in
+ * rank order rounded once, bit-identical to tccl_all_reduce_sum().  Shot 1: rank r's
+ * workgroups reduce share r (numel / world elements) from all buffers into their own buffer;
+ * then the reference's blockwise barrier (triton_barrier.py:39-142: workgroup g of every
+ * rank signals workgroup g of every other rank through slot `g * world + sender` of the
+ * receiver's pad and waits for the same from them); shot 2: every rank copies the other
+ * shares from their owners' buffers.  This is the reduce-scatter + all-gather composition
+ * the reference's slides name for large messages, as one kernel; it moves (3*world - 1)/world
+ * buffers per rank instead of the (world + 1) of a one-shot all-reduce per rank.
+ * 1 <= world <= TCCL_MAX_WORLD; numel % (world * 16 / esize) == 0 (whole vectors per share,
+ * the reduce-scatter's precondition).  signal_pads / pad_bytes / time-outs / residency: as for
+ * tccl_double_tree_all_reduce_pipelined; pad_bytes >= 4 * (world + 1) rounded up to 16 is
+ * enough, larger pads allow more workgroups per rank (cfg->lag and cfg->tile_kib are unused). */
+int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *signal_pads,
+                             size_t pad_bytes, int world, size_t numel, int dtype,
+                             const tccl_pipeline_cfg *cfg, void *stream);
 
 /* HIP-event helpers so a host language without HIP bindings can time launches on the very
  * stream they run on.  No counterpart in the reference (it times with torch.cuda.Event,

@@ -247,7 +247,7 @@ def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, 
     ``pipelined``: one persistent launch in which the ranks' workgroups hand chunks to each
     other through the group's signal pads (the reference kernel's wait/reduce/send design,
     triton_double_tree_allreduce.py:254-335) instead of one launch per tree level.  Check
-    ``double_tree_pipelined_timeouts`` afterwards when a wait may have expired."""
+    ``signal_pad_timeouts`` afterwards when a wait may have expired."""
     like = group.tensors[0].reshape(-1)
     if numel is not None:
         like = like[:numel]
@@ -257,20 +257,50 @@ def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, 
     return _run_double_tree(group, like.numel(), dtype, like, chunk_elems, fused, pipelined, pipeline_cfg)
 
 
-def double_tree_pipelined_timeouts(group: SymmGroup, numel: Optional[int] = None, *, chunk_elems: int = 0) -> int:
-    """Waits of pipelined calls on ``group`` that expired since its pads were last cleared
-    (0 after correct runs).  Synchronises the current stream."""
-    like = group.tensors[0].reshape(-1)
-    if numel is not None:
-        like = like[:numel]
+def signal_pad_timeouts(group: SymmGroup) -> int:
+    """Waits of signalling kernels (pipelined double tree, one-launch two-shot) on ``group``
+    that expired since its pads were last cleared; 0 after correct runs.  Synchronises the
+    current stream."""
     if group.signal_pad_bytes == 0:
         return 0
     count = ctypes.c_uint(0)
-    rc = _lib.load().tccl_double_tree_pipelined_timeouts(
-        group.signal_pads(group.signal_pad_bytes), group.world_size, like.numel(), _sum_dtype(like), chunk_elems,
-        ctypes.byref(count), _stream(like.device))
-    _lib.check("tccl_double_tree_pipelined_timeouts", rc)
+    pads = group.signal_pads(group.signal_pad_bytes)
+    rc = _lib.load().tccl_signal_pad_timeouts(pads[0], group.signal_pad_bytes, ctypes.byref(count),
+                                              _stream(group.tensors[0].device))
+    _lib.check("tccl_signal_pad_timeouts", rc)
     return int(count.value)
+
+
+# Signal pad size the one-launch two-shot asks for: room for 1024 workgroups per rank.
+TWO_SHOT_PAD_BYTES = 4 * (8 * 1024 + 4)
+
+
+def two_shot_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *, with_outputs: bool = True,
+                              pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> Optional[List[torch.Tensor]]:
+    """Two-shot all-reduce of every virtual rank of ``group`` in one launch, in place: every
+    buffer ends up holding the sum (bit-identical to ``one_shot_all_reduce``); with
+    ``with_outputs`` the W results are also written to fresh tensors, which are returned.
+    Shot 1 reduces each rank's share, the reference's blockwise barrier
+    (triton_barrier.py:39-142) separates it from shot 2, which gathers the other shares."""
+    like = group.tensors[0].reshape(-1)
+    if numel is not None:
+        like = like[:numel]
+    dtype = _sum_dtype(like)
+    world = group.world_size
+    assert like.numel() % (_vec_elems(like) * world) == 0, "The number of elements must be 128-bit aligned."
+    lib = _lib.load()
+    outputs = None
+    out_ptrs = None
+    if with_outputs:
+        stacked = torch.empty((world, like.numel()), dtype=like.dtype, device=like.device)
+        outputs = list(stacked.unbind(0))
+        out_ptrs = _lib.ptr_array([int(o.data_ptr()) for o in outputs])
+    pads = group.signal_pads(TWO_SHOT_PAD_BYTES)
+    rc = lib.tccl_two_shot_all_reduce(group.ptr_array, out_ptrs, pads, group.signal_pad_bytes, world, like.numel(),
+                                      dtype, ctypes.byref(pipeline_cfg) if pipeline_cfg is not None else None,
+                                      _stream(like.device))
+    _lib.check("tccl_two_shot_all_reduce", rc)
+    return outputs
 
 
 class DoubleTreePlan:

@@ -54,7 +54,7 @@ def run_and_check(group, want, what, **kw):
     print(f"pipelined: {what} {kw}", flush=True)
     outs = tccl_amd.double_tree_all_reduce_world(group, pipelined=True, **kw)
     chunk = kw.get("chunk_elems", 0)
-    assert tccl_amd.double_tree_pipelined_timeouts(group, chunk_elems=chunk) == 0, f"{what}: a wait expired"
+    assert tccl_amd.signal_pad_timeouts(group) == 0, f"{what}: a wait expired"
     for r in range(group.world_size):
         assert_bit_equal(outs[r], want, f"{what}: output {r}")
         assert_bit_equal(group.tensor(r), want, f"{what}: buffer {r}")
@@ -120,7 +120,7 @@ def test_pipelined_fill_rank(_gpu_hygiene):
     world = 8
     g = upload(_gpu_hygiene, [torch.full((65_536 * 4,), float(r), dtype=torch.bfloat16) for r in range(world)])
     outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg())
-    assert tccl_amd.double_tree_pipelined_timeouts(g) == 0
+    assert tccl_amd.signal_pad_timeouts(g) == 0
     for r in range(world):
         assert outs[r].eq(28).all().item()
 
@@ -139,7 +139,7 @@ def test_pipelined_without_outputs_through_c_abi(_gpu_hygiene):
     rc = lib.tccl_double_tree_all_reduce_pipelined(g.ptr_array, None, pads, g.signal_pad_bytes, world, numel,
                                                    _lib.TCCL_BF16, 0, ctypes.byref(c), s)
     assert rc == 0
-    assert tccl_amd.double_tree_pipelined_timeouts(g) == 0
+    assert tccl_amd.signal_pad_timeouts(g) == 0
     for r in range(world):
         assert_bit_equal(g.tensor(r), want, f"buffer {r}")
 
@@ -159,7 +159,7 @@ def test_pipelined_full_size_properties(_gpu_hygiene):
     want = total.to(torch.bfloat16)       # |sum| <= 64: exact in bf16 at every node
     del total
     outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1 << 20))
-    assert tccl_amd.double_tree_pipelined_timeouts(g) == 0
+    assert tccl_amd.signal_pad_timeouts(g) == 0
     for r in range(world):
         assert torch.equal(outs[r], want), f"output {r}"
         assert torch.equal(g.tensor(r), want), f"buffer {r}"
@@ -177,7 +177,7 @@ def test_pipelined_expired_waits_drain_and_recover(_gpu_hygiene):
     print("pipelined: spin limit 1", flush=True)
     tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1))
     torch.cuda.synchronize()                         # the grid drained
-    expired = tccl_amd.double_tree_pipelined_timeouts(g)
+    expired = tccl_amd.signal_pad_timeouts(g)
     if expired == 0:                                 # every signal happened to be there already
         for r in range(world):
             assert_bit_equal(g.tensor(r), want, f"buffer {r}")
@@ -205,3 +205,113 @@ def test_pipelined_argument_checks(_gpu_hygiene):
     assert call(g8.ptr_array, None, pads, need, 8, 64, _lib.TCCL_BF16, 12, None, None) == _lib.TCCL_EALIGN
     assert call(g8.ptr_array, None, pads, need, 3, 64, _lib.TCCL_BF16, 0, None, None) == _lib.TCCL_EPOW2
     assert call(g8.ptr_array, None, pads, need, 8, 0, _lib.TCCL_BF16, 0, None, None) == 0
+
+
+# ---------------------------------------------------------------- one-launch two-shot all-reduce
+
+def oracle_sum(c_oracle, bufs):
+    if bufs[0].dtype == torch.bfloat16:
+        return from_np_bits(c_oracle.all_reduce_bf16([np_bits(b) for b in bufs]))
+    return torch.from_numpy(c_oracle.all_reduce_f32([b.numpy() for b in bufs]))
+
+
+def two_shot_and_check(group, want, what, **kw):
+    print(f"two-shot: {what} {kw}", flush=True)
+    outs = tccl_amd.two_shot_all_reduce_world(group, **kw)
+    assert tccl_amd.signal_pad_timeouts(group) == 0, f"{what}: a wait expired"
+    for r in range(group.world_size):
+        if outs is not None:
+            assert_bit_equal(outs[r], want, f"{what}: output {r}")
+        assert_bit_equal(group.tensor(r), want, f"{what}: buffer {r}")
+    assert pads_are_zero(group), f"{what}: signal pads not reset"
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
+@pytest.mark.parametrize("vecs_per_share", [1, 3, 1_023, 1_024, 1_025, 70_001])
+def test_two_shot_one_launch_matches_oracle(world, maker, vecs_per_share, _gpu_hygiene, c_oracle):
+    """Every buffer and every output equals the one-shot all-reduce of the oracle, bit for
+    bit: shares of one vector, around one 16 KiB tile (1,024 vectors) and many ragged tiles."""
+    per_vec = 8 if maker is seeded_randn else 4
+    numel = vecs_per_share * per_vec * world
+    bufs = maker(world, numel, seed_base=950)
+    want = oracle_sum(c_oracle, bufs)
+    g = upload(_gpu_hygiene, bufs)
+    two_shot_and_check(g, want, f"W={world} n={numel}", pipeline_cfg=cfg())
+    one = tccl_amd.one_shot_all_reduce(upload(_gpu_hygiene, bufs).tensor(0))
+    assert_bit_equal(one, want, "one-shot kernel agrees")
+
+
+@pytest.mark.parametrize("workgroups", [8, 16, 24, 64, 512, 0])
+@pytest.mark.parametrize("with_outputs", [True, False])
+def test_two_shot_grid_and_in_place_only(workgroups, with_outputs, _gpu_hygiene, c_oracle):
+    world, numel = 8, 8 * 8 * 40_001
+    bufs = seeded_randn(world, numel, seed_base=960)
+    want = oracle_sum(c_oracle, bufs)
+    g = upload(_gpu_hygiene, bufs)
+    two_shot_and_check(g, want, f"wgs={workgroups} outs={with_outputs}", with_outputs=with_outputs,
+                       pipeline_cfg=cfg(workgroups))
+
+
+def test_two_shot_order_sensitive_and_repeats(_gpu_hygiene):
+    """[2^24, 1 x 6, -2^24] sums to 0 only in rank order (fp32); then the same group again with
+    fill(rank) -> 28, without clearing the pads."""
+    world, numel = 8, 4 * 8 * 1_000
+    vals = [2.0 ** 24, 1, 1, 1, 1, 1, 1, -(2.0 ** 24)]
+    g = upload(_gpu_hygiene, [torch.full((numel,), v, dtype=torch.float32) for v in vals])
+    two_shot_and_check(g, torch.zeros(numel, dtype=torch.float32), "rank order", pipeline_cfg=cfg())
+    for r in range(world):
+        g.tensor(r).fill_(float(r))
+    two_shot_and_check(g, torch.full((numel,), 28.0, dtype=torch.float32), "fill(rank)", pipeline_cfg=cfg())
+
+
+def test_two_shot_full_size(_gpu_hygiene):
+    """The headline shape, 8 x 64 MiB bf16: against the one-shot kernel's result."""
+    world, numel = 8, 33_554_432
+    g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    for r in range(world):
+        g.tensor(r).copy_(torch.randn(numel, generator=gen, device=DEV, dtype=torch.float32))
+    want = tccl_amd.one_shot_all_reduce(g.tensor(0))
+    outs = tccl_amd.two_shot_all_reduce_world(g, pipeline_cfg=cfg(spin_limit=1 << 20))
+    assert tccl_amd.signal_pad_timeouts(g) == 0
+    for r in range(world):
+        assert torch.equal(outs[r].view(torch.int16), want.view(torch.int16)), f"output {r}"
+        assert torch.equal(g.tensor(r).view(torch.int16), want.view(torch.int16)), f"buffer {r}"
+    assert pads_are_zero(g)
+
+
+def test_two_shot_expired_barrier_drains_and_recovers(_gpu_hygiene, c_oracle):
+    """Failure handling, forced from the host: with one poll per wait the barrier expires
+    unless every peer happens to be there already; the launch ends either way, and after
+    clearing the pads the group works again."""
+    world, numel = 8, 8 * 8 * 200_000
+    bufs = seeded_randn(world, numel, seed_base=970)
+    want = oracle_sum(c_oracle, bufs)
+    g = upload(_gpu_hygiene, bufs)
+    print("two-shot: spin limit 1", flush=True)
+    tccl_amd.two_shot_all_reduce_world(g, pipeline_cfg=cfg(spin_limit=1))
+    torch.cuda.synchronize()
+    if tccl_amd.signal_pad_timeouts(g) == 0:
+        for r in range(world):
+            assert_bit_equal(g.tensor(r), want, f"buffer {r}")
+        return
+    g.clear_signal_pads()
+    for r, b in enumerate(bufs):
+        g.tensor(r).copy_(b)
+    two_shot_and_check(g, want, "after clearing the pads", pipeline_cfg=cfg())
+
+
+def test_two_shot_argument_checks(_gpu_hygiene):
+    lib = tccl_amd.load_library()
+    g = tccl_amd.empty_world(8, 8 * 8 * 4, torch.bfloat16, DEV)
+    _gpu_hygiene.append(g)
+    pads = g.signal_pads(4096)
+    call = lib.tccl_two_shot_all_reduce
+    assert call(g.ptr_array, None, pads, 4096, 9, 256, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL
+    assert call(g.ptr_array, None, pads, 16, 8, 256, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL   # pad too small
+    assert call(g.ptr_array, None, None, 4096, 8, 256, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL
+    assert call(g.ptr_array, None, pads, 4096, 8, 8 * 9, _lib.TCCL_BF16, None, None) == _lib.TCCL_EALIGN
+    assert call(g.ptr_array, None, pads, 4096, 8, 256, 7, None, None) == _lib.TCCL_EINVAL
+    assert call(g.ptr_array, None, pads, 4096, 8, 0, _lib.TCCL_BF16, None, None) == 0
