@@ -110,6 +110,40 @@ int main(void)
     HIP_OK(hipMemcpy(host, bufs[4], (size_t)N * 2, hipMemcpyDeviceToHost));
     if (!all_equal(host, N, bf16_of_small_int(84), "tree step + copy")) return 4;
 
+    /* the signalling kernels: refill with the ranks, zero-filled pads from hipMalloc + hipMemset */
+    void *pads[W];
+    size_t pad_bytes = tccl_double_tree_signal_pad_bytes(W, N, TCCL_BF16, 0);
+    if (pad_bytes < 4096) pad_bytes = 4096;
+    for (int r = 0; r < W; ++r) {
+        HIP_OK(hipMalloc(&pads[r], pad_bytes));
+        HIP_OK(hipMemset(pads[r], 0, pad_bytes));
+        for (size_t i = 0; i < N; ++i) host[i] = bf16_of_small_int(r);
+        HIP_OK(hipMemcpy(bufs[r], host, (size_t)N * 2, hipMemcpyHostToDevice));
+    }
+    unsigned expired = 1;
+    TCCL_OK_(tccl_double_tree_all_reduce_pipelined(bufs, outs, pads, pad_bytes, W, N, TCCL_BF16, 0, NULL, stream));
+    TCCL_OK_(tccl_signal_pad_timeouts(pads[0], pad_bytes, &expired, stream));
+    if (expired != 0) {
+        fprintf(stderr, "pipelined double tree: %u waits expired\n", expired);
+        return 4;
+    }
+    for (int r = 0; r < W; ++r) {
+        HIP_OK(hipMemcpy(host, outs[r], (size_t)N * 2, hipMemcpyDeviceToHost));
+        if (!all_equal(host, N, sum, "pipelined double-tree output")) return 4;
+    }
+    /* every buffer holds 28 now: the in-place two-shot all-reduce of eight of them gives 224 */
+    TCCL_OK_(tccl_two_shot_all_reduce(bufs, NULL, pads, pad_bytes, W, N, TCCL_BF16, NULL, stream));
+    TCCL_OK_(tccl_signal_pad_timeouts(pads[0], pad_bytes, &expired, stream));
+    if (expired != 0) {
+        fprintf(stderr, "two-shot all-reduce: %u waits expired\n", expired);
+        return 4;
+    }
+    for (int r = 0; r < W; ++r) {
+        HIP_OK(hipMemcpy(host, bufs[r], (size_t)N * 2, hipMemcpyDeviceToHost));
+        if (!all_equal(host, N, bf16_of_small_int(224), "two-shot buffer")) return 4;
+        hipFree(pads[r]);
+    }
+
     /* error codes instead of faults */
     if (tccl_all_reduce_sum((const void *const *)bufs, 9, out, N, TCCL_BF16, stream) != TCCL_EINVAL) return 5;
     if (tccl_all_gather((const void *const *)bufs, W, gathered, 24, stream) != TCCL_EALIGN) return 5;
