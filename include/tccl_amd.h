@@ -198,6 +198,9 @@ int tccl_plan_destroy(tccl_plan *plan);
  * of triton_barrier.py:39-142 (a sender writes into the RECEIVER's pad, the receiver polls
  * its own pad and resets the slot), with one slot per (tree, chunk, sender) so that a send
  * never blocks.  Leaves memory in the same final state as tccl_double_tree_all_reduce().
+ * chunk_elems = elements per pipelining chunk (whole 16-byte vectors); 0 = 128 KiB worth,
+ * halved down to 4 KiB while a tree would have fewer than 256 chunks (a chunk crosses up to
+ * 2*log2(world) dependent steps, so small inputs want many small chunks in flight).
  *
  * signal_pads: HOST array of `world` device pointers (the reference's
  *   symm_mem.signal_pad_ptrs_dev), each to pad_bytes >= tccl_double_tree_signal_pad_bytes()
@@ -211,8 +214,8 @@ int tccl_plan_destroy(tccl_plan *plan);
  *   grid from the occupancy HIP reports, and a device must run only ONE pipelined call at a
  *   time (two overlapping ones can starve each other until they time out). */
 typedef struct {
-    int workgroups;      /* total workgroups (all ranks); 0 = as many as are safely resident at once
-                            (also the upper limit) */
+    int workgroups;      /* total workgroups (all ranks); 0 = four per compute unit; never more than are
+                            safely resident at once */
     int lag;             /* 1 + rounds the down-sweep runs behind the up-sweep; 0 = default (1: none) */
     unsigned spin_limit; /* polls before a wait gives up; 0 = default (about a second) */
     int tile_kib;        /* a workgroup works a chunk in tiles of 32 (default) or 128 KiB */

@@ -200,7 +200,7 @@ def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tenso
 
 
 def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
-                           fused: Optional[bool] = None) -> torch.Tensor:
+                           fused: Optional[bool] = None, pipelined: bool = False) -> torch.Tensor:
     """All-reduce over two complementary binary trees, one per half of the elements.
 
     Mirrors ``double_tree_all_reduce`` (triton_double_tree_allreduce.py:338-370) as its
@@ -216,7 +216,10 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
 
     ``fused``: False = one launch per tree level (the node-step kernels), True = the whole
     tree in one launch (worlds of 2, 4, 8; same values, same final memory), None = the
-    one-launch kernel up to ``FUSED_TREE_MAX_BYTES`` per buffer, the level schedule above."""
+    one-launch kernel up to ``FUSED_TREE_MAX_BYTES`` per buffer, the level schedule above.
+    ``pipelined``: one persistent launch in which the ranks' workgroups wait for, reduce and
+    signal chunks through the group's signal pads -- the reference kernel's own design
+    (worlds of 2, 4, 8)."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
     if spmd.current_rank() is not None:
@@ -227,14 +230,14 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
             group = symm.group
             if turn.first:
                 group.pending_outputs = dict(enumerate(
-                    _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems, fused)))
+                    _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems, fused, pipelined)))
         return group.pending_outputs[symm.rank]
     symm = rendezvous(tensor)
     group = symm.group
     pending = group.pending_outputs.pop(symm.rank, None)
     if pending is not None and pending.shape == tensor.shape:
         return pending
-    outputs = _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems, fused)
+    outputs = _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems, fused, pipelined)
     group.pending_outputs = {r: o for r, o in enumerate(outputs) if r != symm.rank}
     return outputs[symm.rank]
 

@@ -8,7 +8,8 @@ warm-up.  This harness prints the same columns with the unit fixed (GB/s of inpu
 rank, as the reference counts them) plus the algorithmic HBM GB/s, after a warm-up, timed
 with HIP events on the launch stream.
 
-    python -m tccl_amd.harness all_reduce|reduce_scatter|all_gather|double_tree [--world 8] [--max-elems N]
+    python -m tccl_amd.harness all_reduce|reduce_scatter|all_gather|double_tree|double_tree_pipelined|
+                               two_shot|two_shot_world [--world 8] [--max-elems N]
 """
 from __future__ import annotations
 
@@ -22,7 +23,7 @@ REPS = 10          # as in the reference
 def main(argv=None) -> int:
     p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     p.add_argument("op", choices=["all_reduce", "reduce_scatter", "all_gather", "double_tree", "double_tree_plan", "double_tree_fused",
-                                  "two_shot"])
+                                  "double_tree_pipelined", "two_shot", "two_shot_world"])
     p.add_argument("--world", type=int, default=8)
     p.add_argument("--max-elems", type=int, default=256 * 1024 * 1024 // 2,
                    help="largest element count per rank (bf16); halved down to 2,048")
@@ -52,6 +53,13 @@ def main(argv=None) -> int:
         "all_gather": (lambda t: tccl_amd.all_gather(t, world), lambda n: 2 * world * n * 2),
         "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=False), None),
         "double_tree_fused": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=True), None),
+        # one persistent launch, virtual ranks signalling each other per chunk
+        "double_tree_pipelined": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), pipelined=True),
+                                  None),
+        # every rank's all-reduce in place in one launch (reduce own share, barrier, gather the rest)
+        "two_shot_world": (lambda t: tccl_amd.two_shot_all_reduce_world(group, t.numel() // (8 * world) * 8 * world,
+                                                                        with_outputs=False),
+                           lambda n: (3 * world - 1) * n * 2),
     }
 
     def torch_eager(view):
@@ -103,6 +111,9 @@ def main(argv=None) -> int:
             t_ms = ms.value / REPS
             print(f"torch {size * 2} {size * 2 / t_ms / 1e6:.3f} GB/s  ({t_ms * 1e3:.1f} us)", flush=True)
         size //= 2
+    if args.op in ("double_tree_pipelined", "two_shot_world"):
+        expired = tccl_amd.signal_pad_timeouts(group)
+        print(f"expired waits: {expired}", flush=True)
     tccl_amd.unregister(group)
     return 0
 

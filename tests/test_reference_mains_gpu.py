@@ -84,7 +84,7 @@ def test_all_gather_main():
         assert_bit_equal(o, outs[0], "all ranks gather the same")
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fused", [False, True, "pipelined"])
 def test_double_tree_all_reduce_main(fused):
     """triton_double_tree_allreduce.py:373-410: 8,192 seeded elements per rank.  The
     reference compares with the flat bf16 running sum (its kernel never produced the value);
@@ -97,7 +97,10 @@ def test_double_tree_all_reduce_main(fused):
         tensor = spmd.empty_strided_p2p(size=(size,), stride=(1,), dtype=torch.bfloat16, device=device,
                                         group_name="world")
         tensor.copy_(torch.randn(size, dtype=torch.bfloat16, generator=gen))
-        output = tccl_amd.double_tree_all_reduce(tensor, fused=fused)
+        if fused == "pipelined":        # the reference kernel's own design: wait, reduce, send
+            output = tccl_amd.double_tree_all_reduce(tensor, pipelined=True)
+        else:
+            output = tccl_amd.double_tree_all_reduce(tensor, fused=fused)
         return output.cpu(), tensor.cpu()
 
     results = spmd.run(WORLD, main)
