@@ -264,6 +264,21 @@ def main():
             "host_cpus": os.cpu_count(),
             "gpu_matches_cpu_bitwise": bool(same),
         }
+        # the same oracle on one thread (three passes), and what it ran on
+        threads = torch.get_num_threads()
+        torch.set_num_threads(1)
+        one_s, _ = cpu_baseline(torch, bufs_cpu, 0.0)
+        torch.set_num_threads(threads)
+        model = ""
+        try:
+            with open("/proc/cpuinfo") as f:
+                model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), "")
+        except OSError:
+            pass
+        result["cpu_baseline"].update({
+            "one_thread": {"value": round(algo_bytes / one_s / 1e9, 2), "unit": "GB/s",
+                           "ms_per_pass": round(one_s * 1e3, 1)},
+            "cpu_model": model, "torch_version": torch.__version__})
         del bufs_cpu
 
     if not args.no_other_ops:
