@@ -211,8 +211,11 @@ int tccl_plan_destroy(tccl_plan *plan);
  *   always ends; the buffers then hold partial results and the pads must be cleared by the
  *   caller.  tccl_signal_pad_timeouts() reads the count (it synchronises the stream).
  * Every workgroup of the launch must be resident at the same time: the library sizes the
- *   grid from the occupancy HIP reports, and a device must run only ONE pipelined call at a
- *   time (two overlapping ones can starve each other until they time out). */
+ *   grid from the occupancy HIP reports, and a device must run only ONE signalling kernel at
+ *   a time (two overlapping ones can starve each other until they time out).  Calls made by
+ *   one process are kept apart by the library (each launch makes its stream wait for the
+ *   previous signalling kernel of the device, on whatever stream that ran); launches recorded
+ *   into a HIP graph, and other processes on the same GPU, are the caller's to keep apart. */
 typedef struct {
     int workgroups;      /* total workgroups (all ranks); 0 = four per compute unit; never more than are
                             safely resident at once */

@@ -22,7 +22,7 @@
 // Forward progress needs every workgroup of the launch resident at once: the grid is sized
 // from the occupancy the runtime reports for the kernel.  Two such launches that overlap in
 // time on one GPU could each hold half the slots and starve each other until the time-out,
-// so a device runs one pipelined call at a time.
+// so a device runs one signalling kernel at a time (see SignallingLaunch).
 #include <mutex>
 
 #include "host.h"
@@ -32,6 +32,57 @@ namespace tccl {
 
 constexpr int kPipeMaxWorld = TCCL_MAX_WORLD;
 constexpr uint32_t kPipeDefaultSpins = 1u << 21;
+
+// Two signalling kernels that overlap on one GPU could each hold part of the workgroup slots
+// and starve each other until their waits expire.  Launches of this process are therefore
+// chained: each one first makes its stream wait for the previous signalling kernel of the same
+// device (an event wait, no host blocking), whatever stream that one ran on.  A stream that is
+// being captured into a graph is left alone (an outside event cannot be waited for inside a
+// capture); keeping replays of such graphs apart is then the caller's business.
+class SignallingLaunch {
+public:
+    explicit SignallingLaunch(hipStream_t stream) : stream_(stream), lock_(mutex())
+    {
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return;
+        }
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return;
+        hipEvent_t &ev = events()[dev];
+        if (ev == nullptr) {
+            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+                ev = nullptr;
+                return;
+            }
+        } else if (hipStreamWaitEvent(stream, ev, 0) != hipSuccess) {
+            return;
+        }
+        event_ = ev;
+    }
+    // after the kernel has been enqueued
+    void launched()
+    {
+        if (event_ != nullptr) (void)hipEventRecord(event_, stream_);
+    }
+
+private:
+    static constexpr int kMaxDevices = 64;
+    static std::mutex &mutex()
+    {
+        static std::mutex m;
+        return m;
+    }
+    static hipEvent_t *events()
+    {
+        static hipEvent_t e[kMaxDevices] = {};
+        return e;
+    }
+    hipStream_t stream_;
+    std::unique_lock<std::mutex> lock_;
+    hipEvent_t event_ = nullptr;
+};
 
 struct PipeArgs {
     char *buf[kPipeMaxWorld];
@@ -277,9 +328,12 @@ static int launch_pipelined(const PipeArgs &a, int wgs_wanted, int world, size_t
     }
     PipeArgs args = a;
     args.wgs_per_rank = per_rank;
+    SignallingLaunch guard(s);
     hipLaunchKernelGGL((tree_pipelined_kernel<Sum, VECS>), dim3(static_cast<unsigned>(per_rank * world)),
                        dim3(kPhasedBlock), 0, s, args);
-    return hip_code(hipGetLastError());
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) guard.launched();
+    return hip_code(e);
 }
 
 template <class Sum>
@@ -557,9 +611,12 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, hipS
     if (per_rank > fit) per_rank = fit;
     if (per_rank < 1) return TCCL_EINVAL;
     a.wgs_per_rank = static_cast<int>(per_rank);
+    SignallingLaunch guard(s);
     hipLaunchKernelGGL((two_shot_kernel<Sum, W>), dim3(static_cast<unsigned>(per_rank * W)), dim3(kPhasedBlock), 0, s,
                        a);
-    return hip_code(hipGetLastError());
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) guard.launched();
+    return hip_code(e);
 }
 
 template <class Sum>

@@ -315,3 +315,35 @@ def test_two_shot_argument_checks(_gpu_hygiene):
     assert call(g.ptr_array, None, pads, 4096, 8, 8 * 9, _lib.TCCL_BF16, None, None) == _lib.TCCL_EALIGN
     assert call(g.ptr_array, None, pads, 4096, 8, 256, 7, None, None) == _lib.TCCL_EINVAL
     assert call(g.ptr_array, None, pads, 4096, 8, 0, _lib.TCCL_BF16, None, None) == 0
+
+
+def test_signalling_kernels_on_two_streams_are_kept_apart(_gpu_hygiene, c_oracle):
+    """Two signalling kernels at once could starve each other of workgroup slots; the library
+    chains them with an event, so launching a pipelined tree and a two-shot all-reduce on two
+    different streams back to back, several times, still gives exact results and no expired
+    wait."""
+    world, numel = 8, 65_536 * 48
+    bufs_a = seeded_randn(world, numel, seed_base=980)
+    bufs_b = seeded_randn(world, numel, seed_base=990)
+    want_a = torch_ref.double_tree_all_reduce(bufs_a)[0]
+    want_b = oracle_sum(c_oracle, bufs_b)
+    ga, gb = upload(_gpu_hygiene, bufs_a), upload(_gpu_hygiene, bufs_b)
+    ga.signal_pads(1 << 16)
+    gb.signal_pads(1 << 16)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for round_ in range(3):
+        print(f"two streams: round {round_}", flush=True)
+        for r in range(world):
+            ga.tensor(r).copy_(bufs_a[r])
+            gb.tensor(r).copy_(bufs_b[r])
+        torch.cuda.synchronize()
+        with torch.cuda.stream(s1):
+            outs_a = tccl_amd.double_tree_all_reduce_world(ga, pipelined=True, pipeline_cfg=cfg())
+        with torch.cuda.stream(s2):
+            tccl_amd.two_shot_all_reduce_world(gb, with_outputs=False, pipeline_cfg=cfg())
+        torch.cuda.synchronize()
+        assert tccl_amd.signal_pad_timeouts(ga) == 0 and tccl_amd.signal_pad_timeouts(gb) == 0
+        for r in range(world):
+            assert_bit_equal(outs_a[r], want_a, f"tree output {r}")
+            assert_bit_equal(gb.tensor(r), want_b, f"two-shot buffer {r}")
