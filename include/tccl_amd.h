@@ -15,7 +15,10 @@
  *     Every launching entry point can be recorded into a caller's HIP graph.
  *   - ordering between virtual ranks and between tree levels is stream order; this
  *     replaces the reference's signal-pad barrier (triton_barrier.py:39-142) and its
- *     wait/send flags (triton_double_tree_allreduce.py:175-225).
+ *     wait/send flags (triton_double_tree_allreduce.py:175-225).  Two entry points keep the
+ *     device-side protocol instead, between the virtual ranks' workgroups of one launch:
+ *     tccl_double_tree_all_reduce_pipelined() and tccl_two_shot_all_reduce(); they take
+ *     signal pads and are the only ones that need all their workgroups resident at once.
  *   - float sums: each bf16 is widened to fp32, accumulated from +0.0f in the order the
  *     sources are given, and rounded once (round-to-nearest-even) on store.  NaN sign
  *     and payload are not specified.
