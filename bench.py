@@ -479,6 +479,17 @@ def run_sweep(torch, tccl_amd, lib, device):
          expired_waits=tccl_amd.signal_pad_timeouts(g))
     drop(g)
 
+    # every rank's all-reduce in one launch (two-shot with the blockwise barrier), W=8 x 64 MiB
+    g = make_world(tccl_amd, torch, 8, 33_554_432, torch.bfloat16, device)
+    for with_outputs in (False, True):
+        _, dev_ms = time_steps(torch, lib,
+                               lambda: tccl_amd.two_shot_all_reduce_world(g, with_outputs=with_outputs), 20, 5)
+        nbytes = ((3 if not with_outputs else 4) * 8 - 1) * 33_554_432 * 2
+        emit(op="two_shot_all_reduce_all_ranks", world=8, bytes_per_buffer=64 << 20, outputs=with_outputs,
+             avg_us=round(dev_ms * 1e3, 1), gbs=round(nbytes / (dev_ms * 1e-3) / 1e9, 1),
+             expired_waits=tccl_amd.signal_pad_timeouts(g))
+    drop(g)
+
 
 if __name__ == "__main__":
     main()
