@@ -81,6 +81,37 @@ def test_argument_checks_return_codes_without_launching():
     assert lib.tccl_plan_destroy(None) == -1
     assert lib.tccl_event_create(None) == -1
     assert lib.tccl_event_elapsed_ms(None, None, None) == -1
+    # the signalling entry points
+    pads = _lib.ptr_array([0x5000, 0x6000])
+    sz = lib.tccl_double_tree_signal_pad_bytes
+    assert sz(8, 134_217_728, 0, 0) == 65_552            # 2 trees x 1,024 chunks x 8 flags + status, padded to 16
+    assert sz(8, 134_217_728, 0, 65_536 * 2) == 32_784   # 512 chunks per tree
+    assert sz(2, 16, 0, 0) == 32                         # one chunk per tree, two flags each, + status = 5 words
+    assert sz(2, 8, 1, 0) == 32
+    assert sz(3, 64, 0, 0) == 0 and sz(16, 64, 0, 0) == 0 and sz(8, 60, 0, 0) == 0 and sz(8, 64, 9, 0) == 0
+    piped = lib.tccl_double_tree_all_reduce_pipelined
+    assert piped(good, None, pads, 4096, 3, 64, 0, 0, None, None) == -3
+    assert piped(good, None, pads, 4096, 16, 64, 0, 0, None, None) == -1
+    assert piped(good, None, pads, 4096, 2, 60, 0, 0, None, None) == -2
+    assert piped(good, None, pads, 4096, 2, 64, 0, 12, None, None) == -2      # chunk not whole vectors
+    assert piped(good, None, None, 4096, 2, 64, 0, 0, None, None) == -1
+    assert piped(good, None, pads, 0, 2, 64, 0, 0, None, None) == -1          # pads too small
+    assert piped(null, None, pads, 4096, 2, 64, 0, 0, None, None) == -1
+    assert piped(odd, None, pads, 4096, 2, 64, 0, 0, None, None) == -2
+    assert piped(good, None, pads, 4096, 2, 0, 0, 0, None, None) == 0
+    two = lib.tccl_two_shot_all_reduce
+    assert two(good, None, pads, 4096, 0, 64, 0, None, None) == -1
+    assert two(good, None, pads, 4096, 9, 64, 0, None, None) == -1
+    assert two(good, None, pads, 4096, 2, 64, 5, None, None) == -1
+    assert two(good, None, pads, 4096, 2, 24, 0, None, None) == -2            # shares not whole vectors
+    assert two(good, None, pads, 8, 2, 64, 0, None, None) == -1               # pads too small
+    assert two(good, None, pads, 4090, 2, 64, 0, None, None) == -1            # pad size not a multiple of 16
+    assert two(null, None, pads, 4096, 2, 64, 0, None, None) == -1
+    assert two(good, None, pads, 4096, 2, 0, 0, None, None) == 0
+    n = ctypes.c_uint(0)
+    assert lib.tccl_signal_pad_timeouts(None, 4096, ctypes.byref(n), None) == -1
+    assert lib.tccl_signal_pad_timeouts(ctypes.c_void_p(0x5000), 8, ctypes.byref(n), None) == -1
+    assert lib.tccl_signal_pad_timeouts(ctypes.c_void_p(0x5000), 4096, None, None) == -1
 
 
 def test_missing_library_fails_loudly(monkeypatch):
