@@ -347,3 +347,56 @@ def test_signalling_kernels_on_two_streams_are_kept_apart(_gpu_hygiene, c_oracle
         for r in range(world):
             assert_bit_equal(outs_a[r], want_a, f"tree output {r}")
             assert_bit_equal(gb.tensor(r), want_b, f"two-shot buffer {r}")
+
+
+def test_signalling_kernels_can_be_captured_in_a_graph(_gpu_hygiene, c_oracle):
+    """Both signalling entry points recorded into a caller's HIP graph (through
+    torch.cuda.graph), replayed several times with new inputs and an eager signalling call in
+    between; every replay is checked, and the pads are clean after each."""
+    world, numel = 8, 65_536 * 20 + 8 * 8 * 33
+    lib = tccl_amd.load_library()
+    ga = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    gb = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
+    _gpu_hygiene.extend([ga, gb])
+    need = lib.tccl_double_tree_signal_pad_bytes(world, numel, _lib.TCCL_BF16, 0)
+    pads_a, pads_b = ga.signal_pads(max(need, 1 << 15)), gb.signal_pads(1 << 15)
+    outs = torch.empty((world, numel), dtype=torch.bfloat16, device=DEV)
+    out_ptrs = _lib.ptr_array([int(outs[r].data_ptr()) for r in range(world)])
+    c = cfg()
+
+    def enqueue():
+        s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        assert lib.tccl_double_tree_all_reduce_pipelined(ga.ptr_array, out_ptrs, pads_a, ga.signal_pad_bytes, world,
+                                                         numel, _lib.TCCL_BF16, 0, ctypes.byref(c), s) == 0
+        assert lib.tccl_two_shot_all_reduce(gb.ptr_array, None, pads_b, gb.signal_pad_bytes, world, numel,
+                                            _lib.TCCL_BF16, ctypes.byref(c), s) == 0
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue()                                  # warm-up outside the capture (first-use queries happen here)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue()
+    for rep in range(3):
+        print(f"captured signalling kernels: replay {rep}", flush=True)
+        bufs = seeded_randn(world, numel, seed_base=1000 + 10 * rep)
+        for r in range(world):
+            ga.tensor(r).copy_(bufs[r])
+            gb.tensor(r).copy_(bufs[r])
+        outs.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert tccl_amd.signal_pad_timeouts(ga) == 0 and tccl_amd.signal_pad_timeouts(gb) == 0
+        tree_want = torch_ref.double_tree_all_reduce(bufs)[0]
+        flat_want = oracle_sum(c_oracle, bufs)
+        for r in range(world):
+            assert_bit_equal(outs[r], tree_want, f"replay {rep}: tree output {r}")
+            assert_bit_equal(gb.tensor(r), flat_want, f"replay {rep}: two-shot buffer {r}")
+        assert pads_are_zero(ga) and pads_are_zero(gb)
+        # an eager signalling call between replays
+        for r in range(world):
+            gb.tensor(r).copy_(bufs[r])
+        two_shot_and_check(gb, flat_want, f"eager after replay {rep}", with_outputs=False, pipeline_cfg=cfg())
