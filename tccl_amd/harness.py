@@ -57,8 +57,7 @@ def main(argv=None) -> int:
         "double_tree_pipelined": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), pipelined=True),
                                   None),
         # every rank's all-reduce in place in one launch (reduce own share, barrier, gather the rest)
-        "two_shot_world": (lambda t: tccl_amd.two_shot_all_reduce_world(group, t.numel() // (8 * world) * 8 * world,
-                                                                        with_outputs=False),
+        "two_shot_world": (lambda t: tccl_amd.two_shot_all_reduce_world(group, t.numel(), with_outputs=False),
                            lambda n: (3 * world - 1) * n * 2),
     }
 
@@ -79,6 +78,7 @@ def main(argv=None) -> int:
 
     size = args.max_elems
     while size >= 2048:
+        size = size // (8 * world) * (8 * world)     # whole 16-byte vectors per rank share, whatever --max-elems was
         view = tensor[:size]
         if args.op == "double_tree_plan":       # one recorded plan per size, replayed
             plan = tccl_amd.DoubleTreePlan(group, size)
