@@ -376,8 +376,11 @@ def other_ops(torch, tccl_amd, lib, device):
     g = make_world(tccl_amd, torch, 8, 134_217_728, torch.bfloat16, device)
     _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g), 5, 2)
     out["double_tree_w8_256MiB_level_schedule_ms"] = round(ms, 3)
+    _, ms = time_steps(torch, lib,
+                       lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True, chunk_elems=65_536), 5, 2)
+    out["double_tree_w8_256MiB_pipelined_128KiB_chunks_ms"] = round(ms, 3)
     _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True), 5, 2)
-    out["double_tree_w8_256MiB_pipelined_ms"] = round(ms, 3)
+    out["double_tree_w8_256MiB_pipelined_32KiB_chunks_ms"] = round(ms, 3)
     out["double_tree_pipelined_expired_waits"] = tccl_amd.signal_pad_timeouts(g)
     tccl_amd.unregister(g)
     del g
@@ -473,10 +476,12 @@ def run_sweep(torch, tccl_amd, lib, device):
     _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g), 5, 2)
     emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20, schedule="one launch per tree level",
          ms=round(dev_ms, 3))
-    _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True), 5, 2)
-    emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20,
-         schedule="one persistent launch, ranks signal each other per 128 KiB chunk", ms=round(dev_ms, 3),
-         expired_waits=tccl_amd.signal_pad_timeouts(g))
+    for chunk_kib in (128, 32):
+        _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(
+            g, pipelined=True, chunk_elems=chunk_kib * 512), 5, 2)
+        emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20,
+             schedule=f"one persistent launch, ranks signal each other per {chunk_kib} KiB chunk",
+             ms=round(dev_ms, 3), expired_waits=tccl_amd.signal_pad_timeouts(g))
     drop(g)
 
     # every rank's all-reduce in one launch (two-shot with the blockwise barrier), W=8 x 64 MiB

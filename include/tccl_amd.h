@@ -201,9 +201,10 @@ int tccl_plan_destroy(tccl_plan *plan);
  * of triton_barrier.py:39-142 (a sender writes into the RECEIVER's pad, the receiver polls
  * its own pad and resets the slot), with one slot per (tree, chunk, sender) so that a send
  * never blocks.  Leaves memory in the same final state as tccl_double_tree_all_reduce().
- * chunk_elems = elements per pipelining chunk (whole 16-byte vectors); 0 = 128 KiB worth,
- * halved down to 4 KiB while a tree would have fewer than 256 chunks (a chunk crosses up to
- * 2*log2(world) dependent steps, so small inputs want many small chunks in flight).
+ * chunk_elems = elements per pipelining chunk, the unit that is signalled (whole 16-byte
+ * vectors); 0 = 32 KiB worth (the measured optimum for large inputs), halved down to 4 KiB
+ * while a tree would have fewer than 256 chunks (a chunk crosses up to 2*log2(world)
+ * dependent steps, so small inputs want many small chunks in flight).
  *
  * signal_pads: HOST array of `world` device pointers (the reference's
  *   symm_mem.signal_pad_ptrs_dev), each to pad_bytes >= tccl_double_tree_signal_pad_bytes()

@@ -84,7 +84,8 @@ def test_argument_checks_return_codes_without_launching():
     # the signalling entry points
     pads = _lib.ptr_array([0x5000, 0x6000])
     sz = lib.tccl_double_tree_signal_pad_bytes
-    assert sz(8, 134_217_728, 0, 0) == 65_552            # 2 trees x 1,024 chunks x 8 flags + status, padded to 16
+    assert sz(8, 134_217_728, 0, 65_536) == 65_552       # 2 trees x 1,024 chunks x 8 flags + status, padded to 16
+    assert sz(8, 134_217_728, 0, 0) == 262_160           # default: 32 KiB chunks, 4,096 per tree
     assert sz(8, 134_217_728, 0, 65_536 * 2) == 32_784   # 512 chunks per tree
     assert sz(2, 16, 0, 0) == 32                         # one chunk per tree, two flags each, + status = 5 words
     assert sz(2, 8, 1, 0) == 32
