@@ -117,3 +117,62 @@ def test_random_all_gather_and_tree_steps(case, c_oracle):
                                    stream) == 0
     assert_bit_equal(a, d_own, "copy dst0")
     assert_bit_equal(b, d_own, "copy dst1")
+
+
+def _signalling_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+        per_vec = 16 // (2 if dtype == torch.bfloat16 else 4)
+        scale = int(rng.choice([1, 1, 40, 700, 9000, 60000]))
+        nvec = int(rng.integers(1, 2 + 97 * scale))
+        chunk_vecs = int(rng.choice([0, 0, 0, 1, 3, 64, 1000, 2048, 8192, 20000]))
+        pcfg = dict(workgroups=int(rng.choice([0, 0, 0, 8, 24, 100, 333, 1000, 5000])), lag=int(rng.choice([0, 1, 2, 4])),
+                    tile_kib=int(rng.choice([0, 32, 128])))
+        out.append((i, int(rng.choice([2, 4, 8])), int(rng.integers(1, 9)), dtype, nvec * per_vec, chunk_vecs * per_vec,
+                    pcfg))
+    return out
+
+
+@pytest.mark.parametrize("case", _signalling_cases(40, 20240611), ids=lambda c: f"case{c[0]}")
+def test_random_signalling_kernels(case, c_oracle):
+    """The pipelined double tree (random power-of-two world, chunk size, grid, lag, tile) and
+    the one-launch two-shot (random world 1..8, grid) against the oracles, with no expired
+    wait and clean pads afterwards."""
+    i, tree_world, flat_world, dtype, numel, chunk_elems, pcfgd = case
+    print(f"signalling case {i}: {case[1:]}", flush=True)
+    pcfg = _lib.PipelineCfg(spin_limit=1 << 18, **pcfgd)
+    # pipelined double tree
+    bufs = _inputs(tree_world, numel, dtype, 3000 + i)
+    want = torch_ref.double_tree_all_reduce(bufs)[0]
+    g = tccl_amd.empty_world(tree_world, numel, dtype, DEV)
+    try:
+        for r, b in enumerate(bufs):
+            g.tensor(r).copy_(b)
+        outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, chunk_elems=chunk_elems, pipeline_cfg=pcfg)
+        assert tccl_amd.signal_pad_timeouts(g) == 0
+        for r in range(tree_world):
+            assert_bit_equal(outs[r], want, f"case {i}: tree output {r}")
+            assert_bit_equal(g.tensor(r), want, f"case {i}: tree buffer {r}")
+        assert all(int(p.count_nonzero().item()) == 0 for p in g._signal_pads)   # noqa: SLF001
+    finally:
+        tccl_amd.unregister(g)
+    # one-launch two-shot: every share whole vectors
+    per_vec = 16 // bufs[0].element_size()
+    numel2 = max(numel // (per_vec * flat_world), 1) * per_vec * flat_world
+    bufs = _inputs(flat_world, numel2, dtype, 4000 + i)
+    want = _oracle(c_oracle, bufs)
+    g = tccl_amd.empty_world(flat_world, numel2, dtype, DEV)
+    try:
+        for r, b in enumerate(bufs):
+            g.tensor(r).copy_(b)
+        outs = tccl_amd.two_shot_all_reduce_world(g, with_outputs=(i % 2 == 0), pipeline_cfg=pcfg)
+        assert tccl_amd.signal_pad_timeouts(g) == 0
+        for r in range(flat_world):
+            if outs is not None:
+                assert_bit_equal(outs[r], want, f"case {i}: two-shot output {r}")
+            assert_bit_equal(g.tensor(r), want, f"case {i}: two-shot buffer {r}")
+        assert all(int(p.count_nonzero().item()) == 0 for p in g._signal_pads)   # noqa: SLF001
+    finally:
+        tccl_amd.unregister(g)
