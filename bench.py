@@ -191,6 +191,26 @@ def main():
     except RuntimeError as e:            # e.g. not enough free memory for seven more sets
         print(f"rotated measurement skipped: {e}", file=sys.stderr)
 
+    # What the memory system gives the two halves of that launch on their own: a pure read pass
+    # over the same 8 buffers and a pure write pass over one output, same launch shape.  The sum
+    # is a read phase followed by a write burst, so their total is its practical bound here.
+    sink = torch.zeros(4096, dtype=torch.uint8, device=device)
+    probe_out = torch.empty_like(mine)
+    pstream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _, read_ms = time_steps(torch, lib, lambda: lib.tccl_probe_read(group.ptr_array, WORLD, BYTES_PER_BUF,
+                                                                    sink.data_ptr(), pstream), 100, 50)
+    _, write_ms = time_steps(torch, lib, lambda: lib.tccl_probe_write(probe_out.data_ptr(), BYTES_PER_BUF, pstream),
+                             100, 50)
+    ceilings = {
+        "read_8x64MiB_us": round(read_ms * 1e3, 2), "read_gbs": round(WORLD * BYTES_PER_BUF / (read_ms * 1e-3) / 1e9, 1),
+        "write_64MiB_us": round(write_ms * 1e3, 2), "write_gbs": round(BYTES_PER_BUF / (write_ms * 1e-3) / 1e9, 1),
+        "read_pass_plus_write_pass_us": round((read_ms + write_ms) * 1e3, 2),
+        "sum_kernel_us": round(dev_ms * 1e3, 2),
+        "note": "tccl_probe_read / tccl_probe_write: the read half and the write half of the sum kernel on their "
+                "own, same buffers and launch shape, 100 launches each",
+    }
+    del probe_out
+
     # p50 latency at 1 MiB per buffer: prefix views of the same allocations
     lat_numel = LAT_BYTES_PER_BUF // 2
     small = mine[:lat_numel]
@@ -229,6 +249,7 @@ def main():
         "pct_of_peak": round(100.0 * gbs_wall / HBM_PEAK_GBS, 2),
         "rotated_over_8_buffer_sets": None if rot_ms is None else {
             "gbs": round(algo_bytes / (rot_ms * 1e-3) / 1e9, 1), "avg_launch_us": round(rot_ms * 1e3, 2)},
+        "memory_system_ceilings": ceilings,
         "p50_us_at_1MiB": round(p50_us, 2),
         "p99_us_at_1MiB": round(p99_us, 2),
         "p50_us_at_1MiB_c_entry_point_only": round(p50_c_us, 2),

@@ -264,6 +264,19 @@ int tccl_event_synchronize(void *event);
 int tccl_event_elapsed_ms(void *start, void *stop, float *ms_out);
 int tccl_stream_synchronize(void *stream);
 
+/* Measuring kernels: the read half and the write half of the large all-reduce on their
+ * own, with its launch shape (256 lanes, 128 KiB tiles, two workgroups per compute unit, one
+ * launch per resident wave of tiles).  The large sum is a read phase followed by a write
+ * burst, so "time of tccl_probe_read + time of tccl_probe_write" is the bound the memory
+ * system sets for it on the GPU at hand; a benchmark prints it beside the sum's own time.
+ * tccl_probe_read reads and reduces `world` buffers of bytes_per_buffer each (bf16
+ * arithmetic) and stores nothing (`sink`: 4,096 bytes of device memory that receives a
+ * checksum in one case out of 2^32, which is what keeps the loads alive);
+ * tccl_probe_write fills `bytes` at dst with a pattern.  No counterpart in the reference. */
+int tccl_probe_read(const void *const *bufs, int world, size_t bytes_per_buffer, void *sink,
+                    void *stream);
+int tccl_probe_write(void *dst, size_t bytes, void *stream);
+
 /* Device facts used for reporting: compute units, memory clock (kHz), bus width (bits),
  * L2 bytes.  Any pointer may be NULL. */
 int tccl_device_info(int *compute_units, int *mem_clock_khz, int *mem_bus_bits, size_t *l2_bytes);

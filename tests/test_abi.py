@@ -109,6 +109,15 @@ def test_argument_checks_return_codes_without_launching():
     assert two(good, None, pads, 4090, 2, 64, 0, None, None) == -1            # pad size not a multiple of 16
     assert two(null, None, pads, 4096, 2, 64, 0, None, None) == -1
     assert two(good, None, pads, 4096, 2, 0, 0, None, None) == 0
+    assert lib.tccl_probe_read(good, 2, 64, None, None) == -1
+    assert lib.tccl_probe_read(good, 9, 64, out, None) == -1
+    assert lib.tccl_probe_read(null, 2, 64, out, None) == -1
+    assert lib.tccl_probe_read(odd, 2, 64, out, None) == -2
+    assert lib.tccl_probe_read(good, 2, 24, out, None) == -2
+    assert lib.tccl_probe_read(good, 2, 0, out, None) == 0
+    assert lib.tccl_probe_write(None, 64, None) == -1
+    assert lib.tccl_probe_write(out, 24, None) == -2
+    assert lib.tccl_probe_write(out, 0, None) == 0
     n = ctypes.c_uint(0)
     assert lib.tccl_signal_pad_timeouts(None, 4096, ctypes.byref(n), None) == -1
     assert lib.tccl_signal_pad_timeouts(ctypes.c_void_p(0x5000), 8, ctypes.byref(n), None) == -1

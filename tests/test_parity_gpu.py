@@ -772,3 +772,28 @@ def test_plain_c_client():
     proc = subprocess.run([exe], capture_output=True, text=True, timeout=120, env=env)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "c client ok" in proc.stdout
+
+
+def test_probe_kernels_touch_what_they_say(_gpu_hygiene):
+    """The measuring kernels: the read probe stores nothing (sources and sink unchanged, for
+    every world and for ragged sizes), the write probe fills exactly the bytes it is given."""
+    lib = tccl_amd.load_library()
+    for world, nbytes in [(1, 16), (3, 128 * 1024 + 48), (8, 5 * 128 * 1024 * 512 // 4 + 16), (8, 64 << 20)]:
+        numel = nbytes // 2
+        bufs = [torch.randn(numel, dtype=torch.float32, device=DEV).to(torch.bfloat16) for _ in range(world)]
+        before = [b.clone() for b in bufs]
+        sink = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+        ptrs = _lib.ptr_array([b.data_ptr() for b in bufs])
+        assert lib.tccl_probe_read(ptrs, world, nbytes, sink.data_ptr(), stream()) == 0
+        torch.cuda.synchronize()
+        assert int(sink.count_nonzero().item()) == 0
+        for b, want in zip(bufs, before):
+            assert torch.equal(b.view(torch.int16), want.view(torch.int16))
+    for nbytes in [16, 128 * 1024 - 16, 128 * 1024 * 513 + 32, 64 << 20]:
+        guard = 256
+        region = torch.full((nbytes + 2 * guard,), 0xAB, dtype=torch.uint8, device=DEV)
+        assert lib.tccl_probe_write(region.data_ptr() + guard, nbytes, stream()) == 0
+        torch.cuda.synchronize()
+        assert bool((region[:guard] == 0xAB).all()) and bool((region[guard + nbytes:] == 0xAB).all())
+        words = region[guard:guard + nbytes].view(torch.int32)
+        assert bool((words[0::4] == 0x3F803F80).all()) and bool((words[3::4] == 0x3F803F80).all())
