@@ -4,6 +4,10 @@ Each function takes *this rank's* buffer, finds its peers with ``rendezvous`` ex
 the reference's wrappers do, allocates the output with torch and launches one HIP kernel
 (one per tree level for the double tree) through the C ABI on torch's current stream.
 Preconditions are the reference's own assertions, raised before anything is launched.
+
+The ``*_world`` functions run a collective for every virtual rank of a group at once; two of
+them (``double_tree_all_reduce_world(pipelined=True)``, ``two_shot_all_reduce_world``) use
+kernels in which the ranks' workgroups signal each other through the group's signal pads.
 """
 from __future__ import annotations
 

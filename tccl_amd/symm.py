@@ -8,8 +8,8 @@ obtains the table of all W buffer addresses with ``_SymmetricMemory.rendezvous(t
 Here one process owns all W buffers; ``rendezvous`` finds the group a tensor belongs to in
 a process-local registry keyed by the address of the tensor's storage.  Ordering between
 virtual ranks is the order of work on the HIP stream; signal pads (``signal_pad_ptrs_dev``,
-:87) exist only for the one kernel that signals on the device, the pipelined double tree,
-and are allocated when it is first used.
+:87) exist only for the two kernels that signal on the device, the pipelined double tree and
+the one-launch two-shot all-reduce, and are allocated when one of them is first used.
 """
 from __future__ import annotations
 
