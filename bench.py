@@ -395,7 +395,7 @@ def other_ops(torch, tccl_amd, lib, device):
     # whole double-tree all-reduce, W=8 x 256 MiB in 128 KiB chunks (4 GiB touched per call): the level
     # schedule (one launch per tree level) and the pipelined single launch (ranks signal each other per chunk)
     g = make_world(tccl_amd, torch, 8, 134_217_728, torch.bfloat16, device)
-    _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g), 5, 2)
+    _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, fused=False, pipelined=False), 5, 2)
     out["double_tree_w8_256MiB_level_schedule_ms"] = round(ms, 3)
     _, ms = time_steps(torch, lib,
                        lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True, chunk_elems=65_536), 5, 2)
@@ -494,7 +494,7 @@ def run_sweep(torch, tccl_amd, lib, device):
 
     # whole double-tree all-reduce, W=8 x 256 MiB
     g = make_world(tccl_amd, torch, 8, 134_217_728, torch.bfloat16, device)
-    _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g), 5, 2)
+    _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, fused=False, pipelined=False), 5, 2)
     emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20, schedule="one launch per tree level",
          ms=round(dev_ms, 3))
     for chunk_kib in (128, 32):

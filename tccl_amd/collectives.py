@@ -170,8 +170,14 @@ def all_reduce(tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
 FUSED_TREE_MAX_BYTES = 8 << 20
 
 
+# From this many bytes per buffer the pipelined single launch beats the level schedule for
+# worlds of 2, 4 and 8 (W=8 x 256 MiB: 1.58 ms against 1.74 ms; W=4: 0.67 against 0.77 ms);
+# between the two thresholds the level schedule is as fast or faster.
+PIPELINED_TREE_MIN_BYTES = 192 << 20
+
+
 def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tensor,
-                     chunk_elems: int, fused: Optional[bool] = None, pipelined: bool = False,
+                     chunk_elems: int, fused: Optional[bool] = None, pipelined: Optional[bool] = False,
                      pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> List[torch.Tensor]:
     # one allocation for all W outputs (rows are 16-byte aligned: numel is whole vectors)
     stacked = torch.empty((group.world_size,) + tuple(like.shape), dtype=like.dtype, device=like.device)
@@ -180,6 +186,9 @@ def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tenso
     row_bytes = like.numel() * like.element_size()
     first = int(stacked.data_ptr())
     out_ptrs = _lib.ptr_array([first + r * row_bytes for r in range(group.world_size)])
+    if pipelined is None:
+        pipelined = (fused is None and group.world_size in (2, 4, 8)
+                     and numel * like.element_size() >= PIPELINED_TREE_MIN_BYTES)
     if pipelined:
         need = lib.tccl_double_tree_signal_pad_bytes(group.world_size, numel, dtype, chunk_elems)
         if need == 0:
@@ -204,7 +213,7 @@ def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tenso
 
 
 def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
-                           fused: Optional[bool] = None, pipelined: bool = False) -> torch.Tensor:
+                           fused: Optional[bool] = None, pipelined: Optional[bool] = None) -> torch.Tensor:
     """All-reduce over two complementary binary trees, one per half of the elements.
 
     Mirrors ``double_tree_all_reduce`` (triton_double_tree_allreduce.py:338-370) as its
@@ -221,9 +230,10 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
     ``fused``: False = one launch per tree level (the node-step kernels), True = the whole
     tree in one launch (worlds of 2, 4, 8; same values, same final memory), None = the
     one-launch kernel up to ``FUSED_TREE_MAX_BYTES`` per buffer, the level schedule above.
-    ``pipelined``: one persistent launch in which the ranks' workgroups wait for, reduce and
-    signal chunks through the group's signal pads -- the reference kernel's own design
-    (worlds of 2, 4, 8)."""
+    ``pipelined``: True = one persistent launch in which the ranks' workgroups wait for,
+    reduce and signal chunks through the group's signal pads -- the reference kernel's own
+    design (worlds of 2, 4, 8); None = that launch from ``PIPELINED_TREE_MIN_BYTES`` per buffer
+    when ``fused`` is None too, where it is the fastest of the three."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
     if spmd.current_rank() is not None:
@@ -247,7 +257,7 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
 
 
 def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *,
-                                 chunk_elems: int = 0, fused: Optional[bool] = None, pipelined: bool = False,
+                                 chunk_elems: int = 0, fused: Optional[bool] = None, pipelined: Optional[bool] = None,
                                  pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> List[torch.Tensor]:
     """One whole collective for every virtual rank of ``group``; returns the W outputs.
 

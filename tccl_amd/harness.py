@@ -51,7 +51,8 @@ def main(argv=None) -> int:
         "two_shot": (tccl_amd.two_shot_all_reduce, lambda n: (world + 3) * n * 2),
         "reduce_scatter": (tccl_amd.reduce_scatter, lambda n: (world + 1) * (n // world) * 2),
         "all_gather": (lambda t: tccl_amd.all_gather(t, world), lambda n: 2 * world * n * 2),
-        "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=False), None),
+        "double_tree": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=False, pipelined=False),
+                        None),
         "double_tree_fused": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), fused=True), None),
         # one persistent launch, virtual ranks signalling each other per chunk
         "double_tree_pipelined": (lambda t: tccl_amd.double_tree_all_reduce_world(group, t.numel(), pipelined=True),

@@ -723,11 +723,13 @@ def test_double_tree_f32_and_chunk_sizes(_gpu_hygiene, c_oracle):
             assert_bit_equal(outs[r], want, f"chunk={chunk} rank {r}")
 
 
-def test_double_tree_config5_properties(_gpu_hygiene, c_oracle):
+@pytest.mark.parametrize("how", ["level schedule", "default"])
+def test_double_tree_config5_properties(how, _gpu_hygiene, c_oracle):
     """Benchmark shape 5: W=8 x 134,217,728 bf16 (256 MiB each), halves of
     67,108,864 elements, 65,536-element chunks.  Checked by size-independent properties:
     all 8 outputs and all 8 buffers are bit-identical, and windows of the result equal the
-    oracle run on the same windows of the inputs."""
+    oracle run on the same windows of the inputs.  Once with the level schedule and once with
+    whatever the wrapper picks at this size (the pipelined single launch)."""
     world, numel = 8, 134_217_728
     torch.manual_seed(0)
     base = torch.randn(numel, dtype=torch.bfloat16)
@@ -745,7 +747,11 @@ def test_double_tree_config5_properties(_gpu_hygiene, c_oracle):
         a = [g.tensor(r)[lo:lo + n].cpu() for r in range(world)]
         b = [g.tensor(r)[half + lo:half + lo + n].cpu() for r in range(world)]
         samples.append([torch.cat([x, y]) for x, y in zip(a, b)])
-    outs = tccl_amd.double_tree_all_reduce_world(g)
+    if how == "level schedule":
+        outs = tccl_amd.double_tree_all_reduce_world(g, chunk_elems=65_536, fused=False, pipelined=False)
+    else:
+        outs = tccl_amd.double_tree_all_reduce_world(g)
+        assert tccl_amd.signal_pad_timeouts(g) == 0
     for r in range(1, world):
         assert torch.equal(outs[r].view(torch.int16), outs[0].view(torch.int16)), f"output {r}"
     for r in range(world):
