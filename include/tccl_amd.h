@@ -18,7 +18,7 @@
  *     wait/send flags (triton_double_tree_allreduce.py:175-225).  Two entry points keep the
  *     device-side protocol instead, between the virtual ranks' workgroups of one launch:
  *     tccl_double_tree_all_reduce_pipelined() and tccl_two_shot_all_reduce(); they take
- *     signal pads and are the only ones that need all their workgroups resident at once.
+ *     signal pads.
  *   - float sums: each bf16 is widened to fp32, accumulated from +0.0f in the order the
  *     sources are given, and rounded once (round-to-nearest-even) on store.  NaN sign
  *     and payload are not specified.
@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define TCCL_ABI_VERSION 1
+#define TCCL_ABI_VERSION 2
 
 /* Largest number of source buffers one launch can take (virtual world size). */
 #define TCCL_MAX_WORLD 8
@@ -50,6 +50,7 @@ enum {
     TCCL_EINVAL = -1,      /* NULL pointer, world/rank/dtype out of range, size mismatch */
     TCCL_EALIGN = -2,      /* a pointer or a row size is not a multiple of 16 bytes */
     TCCL_EPOW2 = -3,       /* tree world size is not a power of two >= 2 */
+    TCCL_ETIMEOUT = -5,    /* a wait of a signalling kernel expired (reported by host wrappers, never by a launch) */
     TCCL_EHIP_BASE = -1000 /* -(1000 + hipError_t) */
 };
 
@@ -209,24 +210,45 @@ int tccl_plan_destroy(tccl_plan *plan);
  * signal_pads: HOST array of `world` device pointers (the reference's
  *   symm_mem.signal_pad_ptrs_dev), each to pad_bytes >= tccl_double_tree_signal_pad_bytes()
  *   bytes, 16-byte aligned and ZERO-FILLED before the first call.  A completed call leaves
- *   them zero-filled again.  The last 32-bit word of pad 0 (at pad_bytes - 4) counts time-outs.
+ *   them zero-filled again.  The last TCCL_PAD_CONTROL_WORDS 32-bit words of pad 0 are control
+ *   words (counters from which the workgroups draw their places, and -- the very last word,
+ *   at pad_bytes - 4 -- the count of time-outs).
  * Waits are bounded (cfg->spin_limit polls): a workgroup whose signal never comes counts a
  *   time-out and leaves the kernel, and so does everyone who waits for it, so the launch
  *   always ends; the buffers then hold partial results and the pads must be cleared by the
- *   caller.  tccl_signal_pad_timeouts() reads the count (it synchronises the stream).
- * Every workgroup of the launch must be resident at the same time: the library sizes the
- *   grid from the occupancy HIP reports, and a device must run only ONE signalling kernel at
- *   a time (two overlapping ones can starve each other until they time out).  Calls made by
- *   one process are kept apart by the library (each launch makes its stream wait for the
- *   previous signalling kernel of the device, on whatever stream that ran); launches recorded
- *   into a HIP graph, and other processes on the same GPU, are the caller's to keep apart. */
+ *   caller.  tccl_signal_pad_timeouts() reads the count (it synchronises the stream); a caller
+ *   that must not synchronise passes cfg->timeout_flag, a word in pinned host memory that the
+ *   kernel sets to 1 when a wait expires, and looks at it whenever it likes (for instance
+ *   before its next call).
+ * Forward progress.  By default workgroup b of the grid works as rank b / (workgroups per
+ *   rank): that binding is the fastest on large inputs, but a workgroup then waits for
+ *   workgroups anywhere in the grid, so the whole grid must be resident at once.  The library
+ *   never launches more workgroups than the occupancy HIP reports for the kernel; should other
+ *   work keep part of the GPU busy for longer than spin_limit allows, waits expire and are
+ *   reported as above.  With TCCL_PIPE_DRAW_PLACES in cfg->flags forward progress does not
+ *   depend on residency: a workgroup draws its place (rank, index) from a counter when it starts
+ *   to run, and only waits for the workgroups with the same index of the other ranks, whose
+ *   places are drawn next to its own -- they are all running once any later place has been
+ *   drawn, and at most 56 workgroups can ever sit waiting for one that has not started.  Use
+ *   it when these kernels overlap with other kernels on the same GPU; it measured up to 15 %
+ *   slower at 64-256 MiB per buffer on an otherwise idle GPU and the same below 16 MiB.
+ *   Two signalling launches that overlap on one GPU slow each other down; calls made by one
+ *   process are kept apart by the library (each launch makes its stream wait for the previous
+ *   signalling kernel of the device, on whatever stream that ran).  Two launches must never
+ *   share signal pads at the same time. */
+#define TCCL_PAD_CONTROL_WORDS 288
 typedef struct {
-    int workgroups;      /* total workgroups (all ranks); 0 = four per compute unit; never more than are
-                            safely resident at once */
+    int workgroups;      /* total workgroups (all ranks); 0 = chosen by the library */
     int lag;             /* 1 + rounds the down-sweep runs behind the up-sweep; 0 = default (1: none) */
     unsigned spin_limit; /* polls before a wait gives up; 0 = default (about a second) */
     int tile_kib;        /* a workgroup works a chunk in tiles of 32 (default) or 128 KiB */
+    uint32_t *timeout_flag; /* NULL, or a device-visible 32-bit word (pinned host memory, e.g. from
+                               tccl_timeout_flag_create) that is set to 1 when a wait expires */
+    int flags;           /* TCCL_PIPE_* */
+    int pad_;
 } tccl_pipeline_cfg;
+
+#define TCCL_PIPE_DRAW_PLACES 1 /* workgroups draw their places when they start (see above) */
 
 size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int dtype, size_t chunk_elems);
 int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs,
@@ -248,11 +270,18 @@ int tccl_signal_pad_timeouts(const void *pad0, size_t pad_bytes, unsigned *timeo
  * buffers per rank instead of the (world + 1) of a one-shot all-reduce per rank.
  * 1 <= world <= TCCL_MAX_WORLD; numel % (world * 16 / esize) == 0 (whole vectors per share,
  * the reduce-scatter's precondition).  signal_pads / pad_bytes / time-outs / residency: as for
- * tccl_double_tree_all_reduce_pipelined; pad_bytes >= 4 * (world + 1) rounded up to 16 is
+ * tccl_double_tree_all_reduce_pipelined; pad_bytes >= 4 * (world + TCCL_PAD_CONTROL_WORDS) is
  * enough, larger pads allow more workgroups per rank (cfg->lag and cfg->tile_kib are unused). */
 int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *signal_pads,
                              size_t pad_bytes, int world, size_t numel, int dtype,
                              const tccl_pipeline_cfg *cfg, void *stream);
+
+/* A word for tccl_pipeline_cfg.timeout_flag: 32 bits of pinned, device-visible host memory,
+ * zero to begin with.  The caller reads (and zeroes) it through the pointer.  Creating one
+ * allocates host memory; no counterpart in the reference, whose waits spin for ever
+ * (triton_barrier.py:108-118). */
+int tccl_timeout_flag_create(uint32_t **flag_out);
+int tccl_timeout_flag_destroy(uint32_t *flag);
 
 /* HIP-event helpers so a host language without HIP bindings can time launches on the very
  * stream they run on.  No counterpart in the reference (it times with torch.cuda.Event,

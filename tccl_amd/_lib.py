@@ -12,8 +12,8 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtccl_amd.so")
 
-ABI_VERSION = 1
-TCCL_OK, TCCL_EINVAL, TCCL_EALIGN, TCCL_EPOW2 = 0, -1, -2, -3
+ABI_VERSION = 2
+TCCL_OK, TCCL_EINVAL, TCCL_EALIGN, TCCL_EPOW2, TCCL_ETIMEOUT = 0, -1, -2, -3, -5
 MAX_WORLD = 8
 MAX_JOBS = 8
 
@@ -26,6 +26,8 @@ CFG_XCD_CONTIGUOUS = 4
 CFG_TEMPORAL = 8
 CFG_STREAMING = 16
 CFG_PHASED = 32
+
+PIPE_DRAW_PLACES = 1
 
 
 class TcclError(RuntimeError):
@@ -45,7 +47,8 @@ class LaunchCfg(ctypes.Structure):
 class PipelineCfg(ctypes.Structure):
     """Mirror of ``tccl_pipeline_cfg``; any field left 0 is chosen by the library."""
     _fields_ = [("workgroups", ctypes.c_int), ("lag", ctypes.c_int), ("spin_limit", ctypes.c_uint),
-                ("tile_kib", ctypes.c_int)]
+                ("tile_kib", ctypes.c_int), ("timeout_flag", ctypes.POINTER(ctypes.c_uint32)),
+                ("flags", ctypes.c_int), ("pad_", ctypes.c_int)]
 
 
 class NodeJob(ctypes.Structure):
@@ -85,6 +88,8 @@ SIGNATURES = {
     "tccl_probe_write": (_I, [_P, _SZ, _P]),
     "tccl_signal_pad_timeouts": (_I, [_P, _SZ, ctypes.POINTER(ctypes.c_uint), _P]),
     "tccl_two_shot_all_reduce": (_I, [_PP, _PP, _PP, _SZ, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
+    "tccl_timeout_flag_create": (_I, [ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32))]),
+    "tccl_timeout_flag_destroy": (_I, [ctypes.POINTER(ctypes.c_uint32)]),
     "tccl_double_tree_plan_create": (_I, [_PP, _PP, _I, _SZ, _I, _SZ, _PP]),
     "tccl_plan_launch": (_I, [_P, _P]),
     "tccl_plan_destroy": (_I, [_P]),

@@ -47,6 +47,19 @@ def _cfg_ptr(cfg: Optional[_lib.LaunchCfg]):
     return ctypes.byref(cfg) if cfg is not None else None
 
 
+def _signalling_cfg(group: SymmGroup, cfg: Optional[_lib.PipelineCfg], draw_places: bool = False) -> _lib.PipelineCfg:
+    """The caller's tuning values plus the group's time-out flag, so that an expired wait is
+    seen by the next ``check_signals`` without anybody synchronising."""
+    full = _lib.PipelineCfg()
+    if cfg is not None:
+        full.workgroups, full.lag, full.spin_limit, full.tile_kib = cfg.workgroups, cfg.lag, cfg.spin_limit, cfg.tile_kib
+        full.flags = cfg.flags
+    if draw_places:
+        full.flags |= _lib.PIPE_DRAW_PLACES
+    full.timeout_flag = group.timeout_flag
+    return full
+
+
 def _check_out(out: torch.Tensor, shape, like: torch.Tensor) -> torch.Tensor:
     if tuple(out.shape) != tuple(shape) or out.dtype != like.dtype or out.device != like.device \
             or not out.is_contiguous():
@@ -66,6 +79,7 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, out: Optional[torch.Tensor] = N
     lib = _lib.load()
     with spmd.collective():
         symm = rendezvous(tensor)
+        symm.group.check_signals()
         output = torch.empty_like(tensor) if out is None else _check_out(out, tensor.shape, tensor)
         rc = lib.tccl_all_reduce_sum_ex(symm.buffer_ptrs_host, symm.world_size, output.data_ptr(), tensor.numel(),
                                         dtype, _stream(tensor.device), _cfg_ptr(cfg))
@@ -83,6 +97,7 @@ def one_shot_reduce_scatter(tensor: torch.Tensor, *, out: Optional[torch.Tensor]
     lib = _lib.load()
     with spmd.collective():
         symm = rendezvous(tensor)
+        symm.group.check_signals()
         world, rank = symm.world_size, symm.rank
         assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
         per_rank = tensor.numel() // world
@@ -108,6 +123,7 @@ def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, 
     lib = _lib.load()
     with spmd.collective():
         symm = rendezvous(tensor)
+        symm.group.check_signals()
         if world_size is None:
             world_size = symm.world_size
         assert world_size == symm.world_size, "world_size does not match the tensor's symmetric group"
@@ -136,6 +152,7 @@ def two_shot_all_reduce(tensor: torch.Tensor) -> torch.Tensor:
     stream = _stream(tensor.device)
     with spmd.collective():
         symm = rendezvous(tensor)
+        symm.group.check_signals()
         world = symm.world_size
         assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
         per_rank = tensor.numel() // world
@@ -178,7 +195,8 @@ PIPELINED_TREE_MIN_BYTES = 192 << 20
 
 def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tensor,
                      chunk_elems: int, fused: Optional[bool] = None, pipelined: Optional[bool] = False,
-                     pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> List[torch.Tensor]:
+                     pipeline_cfg: Optional[_lib.PipelineCfg] = None, draw_places: bool = False) -> List[torch.Tensor]:
+    group.check_signals()
     # one allocation for all W outputs (rows are 16-byte aligned: numel is whole vectors)
     stacked = torch.empty((group.world_size,) + tuple(like.shape), dtype=like.dtype, device=like.device)
     outputs = list(stacked.unbind(0))
@@ -196,7 +214,7 @@ def _run_double_tree(group: SymmGroup, numel: int, dtype: int, like: torch.Tenso
         pads = group.signal_pads(need)
         rc = lib.tccl_double_tree_all_reduce_pipelined(
             group.ptr_array, out_ptrs, pads, group.signal_pad_bytes, group.world_size, numel, dtype, chunk_elems,
-            ctypes.byref(pipeline_cfg) if pipeline_cfg is not None else None, _stream(like.device))
+            ctypes.byref(_signalling_cfg(group, pipeline_cfg, draw_places)), _stream(like.device))
         _lib.check("tccl_double_tree_all_reduce_pipelined", rc)
         return outputs
     if fused is None:
@@ -225,7 +243,9 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
     A collective is one call per rank.  On one GPU the first rank to call runs the node
     steps of *all* virtual ranks (the ranks' buffers are overwritten with the result, as
     in the reference's design) and gets its output; the other ranks' outputs wait in the
-    group until those ranks call.  A rank calling again starts the next collective.
+    group until those ranks call.  A rank calling again starts the next collective, and so
+    does any rank calling after a buffer of the group has been written to with torch (refilled
+    for the next collective): outputs of an older collective are never handed out then.
 
     ``fused``: False = one launch per tree level (the node-step kernels), True = the whole
     tree in one launch (worlds of 2, 4, 8; same values, same final memory), None = the
@@ -248,30 +268,44 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
         return group.pending_outputs[symm.rank]
     symm = rendezvous(tensor)
     group = symm.group
+    # The outputs of the collective in progress wait in the group for the ranks that have not
+    # called yet.  They are handed out only while every buffer is as that collective left it:
+    # torch counts in-place writes per tensor, so a buffer that has been refilled since (the
+    # next collective's input) makes the cache stale and this call starts a new collective, and
+    # so does a rank that already has its output and calls again.
+    versions = tuple(t._version for t in group.tensors)                 # noqa: SLF001
     pending = group.pending_outputs.pop(symm.rank, None)
-    if pending is not None and pending.shape == tensor.shape:
+    if pending is not None and pending.shape == tensor.shape and versions == group.pending_versions:
         return pending
     outputs = _run_double_tree(group, tensor.numel(), dtype, tensor, chunk_elems, fused, pipelined)
+    group.collective_number += 1
     group.pending_outputs = {r: o for r, o in enumerate(outputs) if r != symm.rank}
+    group.pending_versions = versions
     return outputs[symm.rank]
 
 
 def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *,
                                  chunk_elems: int = 0, fused: Optional[bool] = None, pipelined: Optional[bool] = None,
-                                 pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> List[torch.Tensor]:
+                                 pipeline_cfg: Optional[_lib.PipelineCfg] = None,
+                                 draw_places: bool = False) -> List[torch.Tensor]:
     """One whole collective for every virtual rank of ``group``; returns the W outputs.
 
     ``pipelined``: one persistent launch in which the ranks' workgroups hand chunks to each
     other through the group's signal pads (the reference kernel's wait/reduce/send design,
-    triton_double_tree_allreduce.py:254-335) instead of one launch per tree level.  Check
-    ``signal_pad_timeouts`` afterwards when a wait may have expired."""
+    triton_double_tree_allreduce.py:254-335) instead of one launch per tree level.  Should a
+    wait of that launch expire (it cannot hang: every wait is bounded), the next collective on
+    the group -- or ``group.check_signals()`` -- raises ``TcclError``.
+    ``draw_places``: the launch's workgroups draw their places (rank, index) when they start to
+    run instead of taking them from their hardware index; the launch then makes progress
+    however few of its workgroups are resident at once (for use beside other kernels on the
+    same GPU), at up to 15 % of the speed on large inputs."""
     like = group.tensors[0].reshape(-1)
     if numel is not None:
         like = like[:numel]
     dtype = _sum_dtype(like)
     assert like.numel() % _vec_elems(like) == 0, "The number of elements must be 128-bit aligned."
     group.pending_outputs.clear()
-    return _run_double_tree(group, like.numel(), dtype, like, chunk_elems, fused, pipelined, pipeline_cfg)
+    return _run_double_tree(group, like.numel(), dtype, like, chunk_elems, fused, pipelined, pipeline_cfg, draw_places)
 
 
 def signal_pad_timeouts(group: SymmGroup) -> int:
@@ -289,16 +323,18 @@ def signal_pad_timeouts(group: SymmGroup) -> int:
 
 
 # Signal pad size the one-launch two-shot asks for: room for 1024 workgroups per rank.
-TWO_SHOT_PAD_BYTES = 4 * (8 * 1024 + 4)
+TWO_SHOT_PAD_BYTES = 4 * (8 * 1024 + 288)
 
 
 def two_shot_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *, with_outputs: bool = True,
-                              pipeline_cfg: Optional[_lib.PipelineCfg] = None) -> Optional[List[torch.Tensor]]:
+                              pipeline_cfg: Optional[_lib.PipelineCfg] = None,
+                              draw_places: bool = False) -> Optional[List[torch.Tensor]]:
     """Two-shot all-reduce of every virtual rank of ``group`` in one launch, in place: every
     buffer ends up holding the sum (bit-identical to ``one_shot_all_reduce``); with
     ``with_outputs`` the W results are also written to fresh tensors, which are returned.
     Shot 1 reduces each rank's share, the reference's blockwise barrier
-    (triton_barrier.py:39-142) separates it from shot 2, which gathers the other shares."""
+    (triton_barrier.py:39-142) separates it from shot 2, which gathers the other shares.
+    ``draw_places``: as for ``double_tree_all_reduce_world``."""
     like = group.tensors[0].reshape(-1)
     if numel is not None:
         like = like[:numel]
@@ -312,9 +348,10 @@ def two_shot_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *, 
         stacked = torch.empty((world, like.numel()), dtype=like.dtype, device=like.device)
         outputs = list(stacked.unbind(0))
         out_ptrs = _lib.ptr_array([int(o.data_ptr()) for o in outputs])
+    group.check_signals()
     pads = group.signal_pads(TWO_SHOT_PAD_BYTES)
     rc = lib.tccl_two_shot_all_reduce(group.ptr_array, out_ptrs, pads, group.signal_pad_bytes, world, like.numel(),
-                                      dtype, ctypes.byref(pipeline_cfg) if pipeline_cfg is not None else None,
+                                      dtype, ctypes.byref(_signalling_cfg(group, pipeline_cfg, draw_places)),
                                       _stream(like.device))
     _lib.check("tccl_two_shot_all_reduce", rc)
     return outputs

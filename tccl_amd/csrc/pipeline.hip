@@ -16,13 +16,26 @@
 //    zero-filled is zero-filled again after every completed call (the property that makes the
 //    reference's barrier usable under graph replay);
 //  * every wait is bounded: a workgroup that polls `spin_limit` times without seeing its
-//    signal counts one time-out in the status word and leaves the kernel; whoever waits for
-//    that workgroup then times out the same way, so the grid always drains.
+//    signal counts one time-out in the control words of pad 0 (and raises the caller's host
+//    flag, if it gave one) and leaves the kernel; whoever waits for that workgroup then times
+//    out the same way, so the grid always drains.
 //
-// Forward progress needs every workgroup of the launch resident at once: the grid is sized
-// from the occupancy the runtime reports for the kernel.  Two such launches that overlap in
-// time on one GPU could each hold half the slots and starve each other until the time-out,
-// so a device runs one signalling kernel at a time (see SignallingLaunch).
+// Forward progress.  With the default binding of places to workgroups (by hardware index) a
+// workgroup waits for workgroups anywhere in the grid, so every workgroup of the launch must
+// be resident at once: the grid never exceeds the occupancy the runtime reports for the
+// kernel, and a wait that still expires is reported, never hidden.  With
+// TCCL_PIPE_DRAW_PLACES forward progress does not depend on residency at all: a workgroup
+// takes its place -- which rank it works for and which index g it has among that rank's
+// workgroups -- from a counter it draws from when it starts to run (take_place), so places are
+// handed out in the order in which workgroups really begin to run; and a workgroup only ever
+// waits for the workgroups with the same g of the other ranks, whose places are drawn right
+// before and after its own from the same counter.  So of all groups of W workgroups with
+// equal g that still have work to do, all but at most one per counter (the one being drawn)
+// have every member running: they can finish, their slots go to workgroups that have not
+// started, and those draw the missing places first.  At most 8 * (W - 1) = 56 workgroups can
+// sit waiting for members that have not started, fewer than the slots of any one XCD (32
+// compute units x at least 2 workgroups), so a slot for the next starter is always there,
+// whatever else runs on the GPU.
 #include <mutex>
 
 #include "host.h"
@@ -34,7 +47,8 @@ constexpr int kPipeMaxWorld = TCCL_MAX_WORLD;
 constexpr uint32_t kPipeDefaultSpins = 1u << 21;
 
 // Two signalling kernels that overlap on one GPU could each hold part of the workgroup slots
-// and starve each other until their waits expire.  Launches of this process are therefore
+// and (with places bound by hardware index) starve each other until their waits expire; with
+// drawn places they would only slow each other down.  Launches of this process are therefore
 // chained: each one first makes its stream wait for the previous signalling kernel of the same
 // device (an event wait, no host blocking), whatever stream that one ran on.  A stream that is
 // being captured into a graph is left alone (an outside event cannot be waited for inside a
@@ -97,8 +111,101 @@ struct PipeArgs {
     uint32_t slots;       // chunk slots per tree in a pad (>= both nchunks)
     uint32_t spin_limit;
     int world, wgs_per_rank, lag, tree_height;
-    uint32_t *status; // time-out counter
+    int draw;         // 1 = workgroups draw their places when they start, 0 = places follow the hardware index
+    uint32_t *ctl;    // the control words at the end of pad 0 (place counters ... time-outs)
+    uint32_t *report; // optional word in host memory that is set to 1 when a wait expires
 };
+
+// The last kCtlWords 32-bit words of pad 0: eight place counters (one per list, a cache line
+// apart so that draws from different lists do not queue behind each other in the memory-side
+// atomic unit: draws from one counter take about 10 ns each), the count of lists that have
+// been drawn completely, and -- the very last word -- the count of time-outs.
+constexpr int kCtlStride = 32; // words between two place counters
+constexpr int kCtlListsDone = kNumXcd * kCtlStride;
+constexpr int kCtlWords = kCtlListsDone + kCtlStride;
+constexpr int kCtlTimeouts = kCtlWords - 1;
+constexpr uint32_t kNoPlace = 0xFFFFFFFFu;
+static_assert(kCtlWords == TCCL_PAD_CONTROL_WORDS, "header and library disagree");
+
+// The XCD this wave runs on (0..7): bits 3:0 of the XCC_ID hardware register.  Only a hint
+// for locality; nothing depends on its value being right.
+__device__ __forceinline__ uint32_t xcd_of_this_wave()
+{
+    // s_getreg_b32 hwreg(HW_REG_XCC_ID = 20, offset 0, width 4): id | offset << 6 | (width - 1) << 11
+    return __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & (kNumXcd - 1);
+}
+
+// A workgroup's place in the collective is (rank, g) with g < wgs_per_rank.  Two ways to get it.
+//
+// By hardware index (the default): workgroup b of the grid is rank b / wgs_per_rank, index
+// b % wgs_per_rank.  This is the faster binding on large inputs (which compute unit runs
+// which place matters to the memory system: the same kernel with places bound to workgroups
+// in any other way measured 4-15 % slower at 64-256 MiB per buffer), but a workgroup then
+// waits for workgroups far away in the grid, so the whole grid must be resident at once.
+//
+// By drawing (TCCL_PIPE_DRAW_PLACES): the place is drawn from a counter when the workgroup
+// starts to run.  The places are kept in 8 lists, list x holding the places with g % 8 == x
+// in the order (g, rank); a workgroup draws the next place of the list of the XCD it runs on,
+// and goes on to the following lists when that one has been drawn completely (there are
+// exactly as many workgroups as places, so it always finds one).  Two things follow.
+// (1) Within a list places are drawn in order, so the W places with the same g -- the only
+// workgroups that ever wait for each other -- are drawn one after the other, and once any
+// later place of the list has been drawn all W of them are running.  (2) Workgroups with the
+// same g of all ranks run on the same XCD (as far as the hardware spreads the grid evenly),
+// so a chunk one of them wrote a moment ago is read by the next from that XCD's L2 -- as with
+// the default binding when wgs_per_rank is a multiple of 8.
+// The counters start at zero (the pads are zero-filled before the first call).  The workgroup
+// that draws the last place of a list counts the list as done; the one that completes the
+// count knows that every workgroup of the launch has drawn its place -- nobody will touch
+// the counters again -- and puts all of them back to zero for the next launch.
+__device__ __forceinline__ void take_place(uint32_t *ctl, bool draw, uint32_t world, uint32_t wgs_per_rank, int *rank,
+                                           uint32_t *g, uint32_t *lds_place)
+{
+    if (!draw) {
+        *rank = static_cast<int>(blockIdx.x / wgs_per_rank);
+        *g = blockIdx.x % wgs_per_rank;
+        return;
+    }
+    if (threadIdx.x == 0) {
+        const uint32_t first = xcd_of_this_wave();
+        uint32_t r = 0, gg = kNoPlace; // no place: cannot happen, there are as many places as workgroups
+        for (uint32_t k = 0; k < kNumXcd; ++k) {
+            const uint32_t x = (first + k) & (kNumXcd - 1);
+            if (x >= wgs_per_rank) continue; // an empty list
+            const uint32_t places = world * ((wgs_per_rank - x + kNumXcd - 1) / kNumXcd);
+            const uint32_t u =
+                __hip_atomic_fetch_add(ctl + x * kCtlStride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (u >= places) continue; // that list has been drawn completely
+            gg = x + kNumXcd * (u / world);
+            r = u % world;
+            if (u + 1 == places) {
+                const uint32_t lists = wgs_per_rank < kNumXcd ? wgs_per_rank : kNumXcd;
+                const uint32_t done =
+                    __hip_atomic_fetch_add(ctl + kCtlListsDone, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (done + 1 == lists) {
+                    for (uint32_t y = 0; y < kNumXcd; ++y)
+                        __hip_atomic_store(ctl + y * kCtlStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(ctl + kCtlListsDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            break;
+        }
+        lds_place[0] = r;
+        lds_place[1] = gg;
+    }
+    __syncthreads();
+    // the same for every lane: say so, so that everything derived from them (buffer addresses,
+    // descriptors, loop bounds) stays in scalar registers
+    *rank = __builtin_amdgcn_readfirstlane(static_cast<int>(lds_place[0]));
+    *g = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(lds_place[1])));
+}
+
+// A wait expired: count it, and tell the host if it gave us a word to tell it through.
+__device__ __forceinline__ void report_timeout(uint32_t *ctl, uint32_t *report)
+{
+    __hip_atomic_fetch_add(ctl + kCtlTimeouts, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (report != nullptr) __hip_atomic_store(report, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // Coherence between workgroups on different XCDs (each XCD has its own L2) without flushing
 // or invalidating whole caches: every store of this kernel is a device-scope store (sc1: it
@@ -119,9 +226,10 @@ __device__ __forceinline__ void send_signals(uint32_t *slot0, uint32_t *slot1)
 // Wait until every non-null slot has been raised, and lower it again.  One lane polls (a
 // device-scope load); the result reaches the other lanes through LDS, and the barrier keeps
 // every lane's later loads behind the poll that saw the flag.  Returns false after
-// spin_limit polls without success (counted in *status); the caller then leaves the kernel.
-__device__ __forceinline__ bool wait_signals(uint32_t *slot0, uint32_t *slot1, uint32_t spin_limit, uint32_t *status,
-                                             int *lds_ok)
+// spin_limit polls without success (counted in the control words); the caller then leaves the
+// kernel.
+__device__ __forceinline__ bool wait_signals(uint32_t *slot0, uint32_t *slot1, uint32_t spin_limit, uint32_t *ctl,
+                                             uint32_t *report, int *lds_ok)
 {
     if (slot0 == nullptr && slot1 == nullptr) return true; // uniform over the workgroup
     if (threadIdx.x == 0) {
@@ -141,7 +249,7 @@ __device__ __forceinline__ bool wait_signals(uint32_t *slot0, uint32_t *slot1, u
             }
             if (ok) __hip_atomic_store(s, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (!ok) __hip_atomic_fetch_add(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!ok) report_timeout(ctl, report);
         *lds_ok = ok ? 1 : 0;
     }
     __syncthreads();
@@ -197,7 +305,7 @@ __device__ __forceinline__ bool up_step(const PipeArgs &a, int rank, int t, uint
     // children that are leaves have nothing to signal: their buffers are the inputs
     uint32_t *w0 = (c0 >= 0 && a.height[t][c0] > 0) ? a.pad[rank] + slot + c0 : nullptr;
     uint32_t *w1 = (c1 >= 0 && a.height[t][c1] > 0) ? a.pad[rank] + slot + c1 : nullptr;
-    if (!wait_signals(w0, w1, a.spin_limit, a.status, lds_ok)) return false;
+    if (!wait_signals(w0, w1, a.spin_limit, a.ctl, a.report, lds_ok)) return false;
 
     const size_t off = a.half_off[t] + static_cast<size_t>(c) * a.chunk_bytes;
     const size_t left = a.half_bytes[t] - static_cast<size_t>(c) * a.chunk_bytes;
@@ -239,7 +347,7 @@ __device__ __forceinline__ bool down_step(const PipeArgs &a, int rank, int t, ui
     if (h == a.tree_height) return true; // the extra node already holds and has written the result
     const int parent = a.nbr[t][rank][0], c0 = a.nbr[t][rank][1], c1 = a.nbr[t][rank][2];
     const uint32_t slot = (static_cast<uint32_t>(t) * a.slots + c) * a.world;
-    if (!wait_signals(a.pad[rank] + slot + parent, nullptr, a.spin_limit, a.status, lds_ok)) return false;
+    if (!wait_signals(a.pad[rank] + slot + parent, nullptr, a.spin_limit, a.ctl, a.report, lds_ok)) return false;
 
     const size_t off = a.half_off[t] + static_cast<size_t>(c) * a.chunk_bytes;
     const size_t left = a.half_bytes[t] - static_cast<size_t>(c) * a.chunk_bytes;
@@ -261,14 +369,11 @@ __device__ __forceinline__ bool down_step(const PipeArgs &a, int rank, int t, ui
 // (i - lag)-th.  Every rank's workgroup g walks the same chunks in the same order, and a
 // step only waits for steps of the same chunk that sit at the same or an earlier place in
 // the other ranks' order (up-sweep: lower tree levels; down-sweep: the levels above, ending
-// at the extra node's up-sweep step), so with all workgroups resident nothing waits in a
-// circle.
+// at the extra node's up-sweep step), so among the workgroups with the same g nothing waits in
+// a circle, and those are the only workgroups a workgroup ever waits for (see take_place).
 template <class Sum, int VECS>
-__global__ void __launch_bounds__(kPhasedBlock) tree_pipelined_kernel(PipeArgs a)
+__device__ __forceinline__ void tree_pipelined_walk(const PipeArgs &a, int rank, uint32_t g, int *lds_ok)
 {
-    __shared__ int lds_ok;
-    const int rank = static_cast<int>(blockIdx.x) / a.wgs_per_rank;
-    const uint32_t g = blockIdx.x % a.wgs_per_rank;
     const uint32_t G = a.wgs_per_rank;
     const uint32_t most = a.nchunks[0] > a.nchunks[1] ? a.nchunks[0] : a.nchunks[1];
     if (g >= most) return;
@@ -278,14 +383,25 @@ __global__ void __launch_bounds__(kPhasedBlock) tree_pipelined_kernel(PipeArgs a
         if (i < rounds) {
             const uint32_t c = g + i * G;
             for (int t = 0; t < 2; ++t)
-                if (c < a.nchunks[t] && !up_step<Sum, VECS>(a, rank, t, c, &lds_ok)) return;
+                if (c < a.nchunks[t] && !up_step<Sum, VECS>(a, rank, t, c, lds_ok)) return;
         }
         if (i >= lag) {
             const uint32_t c = g + (i - lag) * G;
             for (int t = 0; t < 2; ++t)
-                if (c < a.nchunks[t] && !down_step<VECS>(a, rank, t, c, &lds_ok)) return;
+                if (c < a.nchunks[t] && !down_step<VECS>(a, rank, t, c, lds_ok)) return;
         }
     }
+}
+
+template <class Sum, int VECS>
+__global__ void __launch_bounds__(kPhasedBlock) tree_pipelined_kernel(PipeArgs a)
+{
+    __shared__ int lds_ok;
+    __shared__ uint32_t lds_place[2];
+    int rank;
+    uint32_t g;
+    take_place(a.ctl, a.draw != 0, a.world, a.wgs_per_rank, &rank, &g, lds_place);
+    if (g != kNoPlace) tree_pipelined_walk<Sum, VECS>(a, rank, g, &lds_ok);
 }
 
 // Workgroups per rank for `units` units of work (chunks, tiles) per rank, at most `most`.
@@ -323,10 +439,11 @@ static int resident_workgroups()
             hipSuccess ||
         per_cu < 1)
         return 0;
-    // Never count on a compute unit's last wave slots: a grid sized to all eight waves per
-    // SIMD that the occupancy query reports did not become resident as a whole on MI355X
-    // (its waits expired), six per compute unit and fewer always did.
-    if (per_cu > 6) per_cu = 6;
+    // The hardware hands a grid's workgroups to the 8 XCDs round-robin and, inside an XCD, to its
+    // 32 compute units round-robin (read back from the hardware-id register of every workgroup
+    // of grids of 4 and 6 per unit: every unit got exactly its share), so a grid of
+    // per_cu * units workgroups is resident as a whole once earlier work has left the units.
+    // With the registers these kernels need (94 to 215 per lane) that is 5, 4 or 2 per unit.
     return per_cu * compute_units();
 }
 
@@ -412,8 +529,8 @@ extern "C" size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int
 {
     PipeGeometry g;
     if (pipe_geometry(world, numel, dtype, chunk_elems, &g) != TCCL_OK) return 0;
-    // two trees x slots x world flags, then the status word; rounded up to 16 bytes
-    const size_t words = 2 * g.slots * static_cast<size_t>(world) + 1;
+    // two trees x slots x world flags, then the control words; rounded up to 16 bytes
+    const size_t words = 2 * g.slots * static_cast<size_t>(world) + kCtlWords;
     return (words * sizeof(uint32_t) + 15) / 16 * 16;
 }
 
@@ -460,7 +577,9 @@ extern "C" int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *co
     a.chunk_bytes = static_cast<uint32_t>(g.chunk_bytes);
     a.slots = static_cast<uint32_t>(g.slots);
     a.world = world;
-    a.status = a.pad[0] + pad_bytes / sizeof(uint32_t) - 1; // the last word of pad 0
+    a.draw = (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
+    a.ctl = a.pad[0] + pad_bytes / sizeof(uint32_t) - kCtlWords; // the last words of pad 0
+    a.report = cfg ? cfg->timeout_flag : nullptr;
     a.spin_limit = (cfg && cfg->spin_limit > 0) ? cfg->spin_limit : kPipeDefaultSpins;
     a.lag = (cfg && cfg->lag > 0) ? cfg->lag - 1 : 0; // cfg->lag is 1-based so that 0 means "default"
     if (a.lag > 64) a.lag = 64;
@@ -495,7 +614,9 @@ struct TwoShotArgs {
     size_t share_bytes; // bytes of one rank's share (multiple of 16)
     uint32_t spin_limit;
     int world, wgs_per_rank;
-    uint32_t *status;
+    int draw;         // 1 = workgroups draw their places when they start, 0 = places follow the hardware index
+    uint32_t *ctl;    // control words at the end of pad 0 (place counters ... time-outs)
+    uint32_t *report; // optional host word set to 1 when a wait expires
 };
 
 // The reference's blockwise barrier (triton_barrier.py:39-142) between the workgroups with
@@ -504,7 +625,7 @@ struct TwoShotArgs {
 // lowers again (each slot has one writer and one reader, so the reference's compare-and-swap
 // loops become a store and a polling load).  Everything the workgroup stored before the
 // barrier is visible to its peers' device-scope loads after it.  Returns false when a wait
-// expired (counted in *status).
+// expired (counted in the control words).
 __device__ __forceinline__ bool blockwise_barrier(const TwoShotArgs &a, int rank, uint32_t g, int *lds_ok)
 {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -526,7 +647,7 @@ __device__ __forceinline__ bool blockwise_barrier(const TwoShotArgs &a, int rank
         if (ok)
             __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else
-            __hip_atomic_fetch_add(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            report_timeout(a.ctl, a.report);
         if (!ok) *lds_ok = 0; // any lane that failed clears the flag
     }
     __syncthreads();
@@ -547,16 +668,13 @@ __device__ __forceinline__ bool blockwise_barrier(const TwoShotArgs &a, int rank
 constexpr int kTwoShotVecs = 4;
 
 template <class Sum, int W>
-__global__ void __launch_bounds__(kPhasedBlock) two_shot_kernel(TwoShotArgs a)
+__device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, uint32_t g, int &lds_ok)
 {
     constexpr int VECS = kTwoShotVecs;
-    __shared__ int lds_ok;
     constexpr int U = PhasedUnroll<W>::value < VECS ? PhasedUnroll<W>::value : VECS;
     constexpr int KMAX = VECS / U;
     constexpr uint32_t span = kPhasedBlock * U * kVecBytes;
     constexpr uint32_t tile_bytes = kPhasedBlock * VECS * kVecBytes;
-    const int rank = static_cast<int>(blockIdx.x) / a.wgs_per_rank;
-    const uint32_t g = blockIdx.x % a.wgs_per_rank;
     const uint32_t G = a.wgs_per_rank;
     if (threadIdx.x == 0) lds_ok = 1;
     // (the barrier's first __syncthreads orders this store before any lane's clear)
@@ -609,6 +727,17 @@ __global__ void __launch_bounds__(kPhasedBlock) two_shot_kernel(TwoShotArgs a)
 }
 
 template <class Sum, int W>
+__global__ void __launch_bounds__(kPhasedBlock) two_shot_kernel(TwoShotArgs a)
+{
+    __shared__ int lds_ok;
+    __shared__ uint32_t lds_place[2];
+    int rank;
+    uint32_t g;
+    take_place(a.ctl, a.draw != 0, W, a.wgs_per_rank, &rank, &g, lds_place);
+    if (g != kNoPlace) two_shot_body<Sum, W>(a, rank, g, lds_ok);
+}
+
+template <class Sum, int W>
 static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, hipStream_t s)
 {
     static std::once_flag once;
@@ -618,13 +747,13 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, hipS
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, two_shot_kernel<Sum, W>, kPhasedBlock, 0) ==
                 hipSuccess &&
             per_cu >= 1)
-            resident = (per_cu > 6 ? 6 : per_cu) * compute_units();
+            resident = per_cu * compute_units();
     });
     if (resident < W) return hip_code(hipErrorLaunchOutOfResources);
     constexpr size_t tile_bytes = static_cast<size_t>(kPhasedBlock) * kTwoShotVecs * kVecBytes;
     const size_t tiles = (a.share_bytes + tile_bytes - 1) / tile_bytes;
-    // one slot per (workgroup index, sender) in every pad; the last word of pad 0 is the status
-    const size_t fit = (pad_words - 1) / W;
+    // one slot per (workgroup index, sender) in every pad; the last words of pad 0 are the control words
+    const size_t fit = (pad_words - kCtlWords) / W;
     if (fit < 1) return TCCL_EINVAL;
     size_t per_rank;
     if (wgs_wanted > 0) {
@@ -661,34 +790,83 @@ static int launch_two_shot_world(const TwoShotArgs &a, int wgs_wanted, size_t pa
     }
 }
 
+// Argument checks shared by the two entry points of the two-shot all-reduce (everything but
+// the signal pads).  TCCL_OK means "launch"; *nothing_to_do is set for an empty input.
+static int two_shot_check(void *const *bufs, void *const *outs, int world, size_t numel, int dtype, bool *nothing_to_do)
+{
+    *nothing_to_do = false;
+    const int esize = dtype_size(dtype);
+    if (esize == 0 || bufs == nullptr || world < 1 || world > TCCL_MAX_WORLD) return TCCL_EINVAL;
+    const size_t per_vec = kVecBytes / esize;
+    if (numel % (per_vec * world) != 0) return TCCL_EALIGN; // every share is whole vectors
+    for (int r = 0; r < world; ++r) {
+        if (bufs[r] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(bufs[r]) || (outs && !aligned16(outs[r]))) return TCCL_EALIGN;
+    }
+    *nothing_to_do = numel == 0;
+    return TCCL_OK;
+}
+
+// The launch itself: `pads` are the W signal pads (device addresses), each of pad_bytes.
+static int two_shot_launch(void *const *bufs, void *const *outs, uint32_t *const *pads, size_t pad_bytes, int world,
+                           size_t numel, int dtype, const tccl_pipeline_cfg *cfg, hipStream_t s)
+{
+    TwoShotArgs a = {};
+    for (int r = 0; r < world; ++r) {
+        a.buf[r] = static_cast<char *>(bufs[r]);
+        a.out[r] = outs ? static_cast<char *>(outs[r]) : nullptr;
+        a.pad[r] = pads[r];
+    }
+    a.share_bytes = numel / world * dtype_size(dtype);
+    a.world = world;
+    a.spin_limit = (cfg && cfg->spin_limit > 0) ? cfg->spin_limit : kPipeDefaultSpins;
+    const size_t pad_words = pad_bytes / sizeof(uint32_t);
+    a.ctl = a.pad[0] + pad_words - kCtlWords;
+    a.report = cfg ? cfg->timeout_flag : nullptr;
+    a.draw = (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
+    const int wgs = cfg ? cfg->workgroups : 0;
+    return dtype == TCCL_BF16 ? launch_two_shot_world<Bf16Sum>(a, wgs, pad_words, s)
+                              : launch_two_shot_world<F32Sum>(a, wgs, pad_words, s);
+}
+
 } // namespace tccl
 
 extern "C" int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *signal_pads,
                                         size_t pad_bytes, int world, size_t numel, int dtype,
                                         const tccl_pipeline_cfg *cfg, void *stream)
 {
-    const int esize = dtype_size(dtype);
-    if (esize == 0 || bufs == nullptr || signal_pads == nullptr || world < 1 || world > TCCL_MAX_WORLD)
+    if (signal_pads == nullptr || world < 1 || world > TCCL_MAX_WORLD) return TCCL_EINVAL;
+    if (pad_bytes % 16 != 0 || pad_bytes < (static_cast<size_t>(world) + kCtlWords) * sizeof(uint32_t))
         return TCCL_EINVAL;
-    if (pad_bytes % 16 != 0 || pad_bytes < (static_cast<size_t>(world) + 1) * sizeof(uint32_t)) return TCCL_EINVAL;
-    const size_t per_vec = kVecBytes / esize;
-    if (numel % (per_vec * world) != 0) return TCCL_EALIGN; // every share is whole vectors
-    TwoShotArgs a = {};
+    bool nothing = false;
+    const int rc = two_shot_check(bufs, outs, world, numel, dtype, &nothing);
+    if (rc != TCCL_OK) return rc;
+    uint32_t *pads[TCCL_MAX_WORLD];
     for (int r = 0; r < world; ++r) {
-        if (bufs[r] == nullptr || signal_pads[r] == nullptr) return TCCL_EINVAL;
-        if (!aligned16(bufs[r]) || !aligned16(signal_pads[r]) || (outs && !aligned16(outs[r]))) return TCCL_EALIGN;
-        a.buf[r] = static_cast<char *>(bufs[r]);
-        a.out[r] = outs ? static_cast<char *>(outs[r]) : nullptr;
-        a.pad[r] = static_cast<uint32_t *>(signal_pads[r]);
+        if (signal_pads[r] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(signal_pads[r])) return TCCL_EALIGN;
+        pads[r] = static_cast<uint32_t *>(signal_pads[r]);
     }
-    if (numel == 0) return TCCL_OK;
-    a.share_bytes = numel / world * esize;
-    a.world = world;
-    a.spin_limit = (cfg && cfg->spin_limit > 0) ? cfg->spin_limit : kPipeDefaultSpins;
-    const size_t pad_words = pad_bytes / sizeof(uint32_t);
-    a.status = a.pad[0] + pad_words - 1;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const int wgs = cfg ? cfg->workgroups : 0;
-    return dtype == TCCL_BF16 ? launch_two_shot_world<Bf16Sum>(a, wgs, pad_words, s)
-                              : launch_two_shot_world<F32Sum>(a, wgs, pad_words, s);
+    if (nothing) return TCCL_OK;
+    return two_shot_launch(bufs, outs, pads, pad_bytes, world, numel, dtype, cfg, static_cast<hipStream_t>(stream));
+}
+
+// A 32-bit word in pinned host memory that the GPU can write: a caller without HIP bindings
+// gets the `timeout_flag` of tccl_pipeline_cfg from here and reads it through the pointer.
+extern "C" int tccl_timeout_flag_create(uint32_t **flag_out)
+{
+    if (flag_out == nullptr) return TCCL_EINVAL;
+    *flag_out = nullptr;
+    void *p = nullptr;
+    const hipError_t e = hipHostMalloc(&p, 64, hipHostMallocMapped | hipHostMallocCoherent);
+    if (e != hipSuccess) return hip_code(e);
+    *static_cast<volatile uint32_t *>(p) = 0u;
+    *flag_out = static_cast<uint32_t *>(p);
+    return TCCL_OK;
+}
+
+extern "C" int tccl_timeout_flag_destroy(uint32_t *flag)
+{
+    if (flag == nullptr) return TCCL_EINVAL;
+    return hip_code(hipHostFree(flag));
 }

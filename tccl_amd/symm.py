@@ -62,6 +62,12 @@ class SymmGroup:
         self.pending_outputs: Dict[int, torch.Tensor] = {}
         self._signal_pads: List[torch.Tensor] = []
         self._signal_pad_array: Optional[ctypes.Array] = None
+        # a word of pinned host memory that a signalling kernel sets when one of its waits expires
+        self._timeout_flag = None
+        # number of the double-tree collective whose outputs `pending_outputs` holds, and torch's
+        # write counters of the W buffers when it ran
+        self.collective_number = 0
+        self.pending_versions: Tuple[int, ...] = ()
 
     def signal_pads(self, nbytes: int) -> ctypes.Array:
         """Host array of W device addresses of zero-filled signal pads of at least ``nbytes``
@@ -69,6 +75,7 @@ class SymmGroup:
         pads are created on first use and replaced by larger ones when needed; the kernels
         that use them leave them zero-filled."""
         if not self._signal_pads or self._signal_pads[0].numel() < nbytes:
+            self.check_signals()            # the old pads' time-out count goes away with them
             device = self.tensors[0].device
             self._signal_pads = [torch.zeros(nbytes, dtype=torch.uint8, device=device)
                                  for _ in range(self.world_size)]
@@ -79,6 +86,35 @@ class SymmGroup:
         """Zero the pads again (needed only after a call that reported time-outs)."""
         for p in self._signal_pads:
             p.zero_()
+
+    @property
+    def timeout_flag(self):
+        """``POINTER(c_uint32)`` to this group's word of pinned host memory; the signalling
+        kernels launched for the group set it to 1 when a wait expires.  Created on first use."""
+        if self._timeout_flag is None:
+            flag = ctypes.POINTER(ctypes.c_uint32)()
+            _lib.check("tccl_timeout_flag_create", _lib.load().tccl_timeout_flag_create(ctypes.byref(flag)))
+            self._timeout_flag = flag
+            weakref.finalize(self, _lib.load().tccl_timeout_flag_destroy, flag)
+        return self._timeout_flag
+
+    def check_signals(self) -> None:
+        """Raise ``TcclError`` (code ``TCCL_ETIMEOUT``) if a wait of a signalling kernel launched
+        for this group has expired since the last check: that collective left partial results
+        in the buffers and its outputs.  Costs one read of host memory, no synchronisation, so
+        every collective on the group calls it first; after a time-out it waits for the device,
+        zeroes the pads and the flag (the group is usable again) and raises."""
+        if self._timeout_flag is None or self._timeout_flag[0] == 0:
+            return
+        torch.cuda.synchronize(self.tensors[0].device)
+        self.clear_signal_pads()
+        torch.cuda.synchronize(self.tensors[0].device)
+        self._timeout_flag[0] = 0
+        self.pending_outputs.clear()
+        raise _lib.TcclError("a signalling collective on this group", _lib.TCCL_ETIMEOUT,
+                             "a wait expired (workgroups it depended on did not run in time): the buffers and "
+                             "outputs of that collective hold partial results; pads cleared, the group can be "
+                             "used again")
 
     @property
     def signal_pad_bytes(self) -> int:

@@ -84,11 +84,12 @@ def test_argument_checks_return_codes_without_launching():
     # the signalling entry points
     pads = _lib.ptr_array([0x5000, 0x6000])
     sz = lib.tccl_double_tree_signal_pad_bytes
-    assert sz(8, 134_217_728, 0, 65_536) == 65_552       # 2 trees x 1,024 chunks x 8 flags + status, padded to 16
-    assert sz(8, 134_217_728, 0, 0) == 262_160           # default: 32 KiB chunks, 4,096 per tree
-    assert sz(8, 134_217_728, 0, 65_536 * 2) == 32_784   # 512 chunks per tree
-    assert sz(2, 16, 0, 0) == 32                         # one chunk per tree, two flags each, + status = 5 words
-    assert sz(2, 8, 1, 0) == 32
+    ctl = 288 * 4                                        # control words at the end of a pad
+    assert sz(8, 134_217_728, 0, 65_536) == 65_536 + ctl       # 2 trees x 1,024 chunks x 8 flags
+    assert sz(8, 134_217_728, 0, 0) == 262_144 + ctl           # default: 32 KiB chunks, 4,096 per tree
+    assert sz(8, 134_217_728, 0, 65_536 * 2) == 32_768 + ctl   # 512 chunks per tree
+    assert sz(2, 16, 0, 0) == 16 + ctl                         # one chunk per tree, two flags each
+    assert sz(2, 8, 1, 0) == 16 + ctl
     assert sz(3, 64, 0, 0) == 0 and sz(16, 64, 0, 0) == 0 and sz(8, 60, 0, 0) == 0 and sz(8, 64, 9, 0) == 0
     piped = lib.tccl_double_tree_all_reduce_pipelined
     assert piped(good, None, pads, 4096, 3, 64, 0, 0, None, None) == -3
@@ -105,10 +106,11 @@ def test_argument_checks_return_codes_without_launching():
     assert two(good, None, pads, 4096, 9, 64, 0, None, None) == -1
     assert two(good, None, pads, 4096, 2, 64, 5, None, None) == -1
     assert two(good, None, pads, 4096, 2, 24, 0, None, None) == -2            # shares not whole vectors
-    assert two(good, None, pads, 8, 2, 64, 0, None, None) == -1               # pads too small
+    assert two(good, None, pads, 1152, 2, 64, 0, None, None) == -1            # pads too small
     assert two(good, None, pads, 4090, 2, 64, 0, None, None) == -1            # pad size not a multiple of 16
     assert two(null, None, pads, 4096, 2, 64, 0, None, None) == -1
     assert two(good, None, pads, 4096, 2, 0, 0, None, None) == 0
+    assert lib.tccl_timeout_flag_create(None) == -1 and lib.tccl_timeout_flag_destroy(None) == -1
     assert lib.tccl_probe_read(good, 2, 64, None, None) == -1
     assert lib.tccl_probe_read(good, 9, 64, out, None) == -1
     assert lib.tccl_probe_read(null, 2, 64, out, None) == -1
@@ -157,9 +159,10 @@ def test_struct_layouts_match_the_header(tmp_path):
         '         offsetof(tccl_launch_cfg, tile_iters), offsetof(tccl_launch_cfg, flags));\n'
         '  printf("%zu %zu %zu %zu %zu\\n", sizeof(tccl_node_job), offsetof(tccl_node_job, src),\n'
         '         offsetof(tccl_node_job, dst), offsetof(tccl_node_job, numel), offsetof(tccl_node_job, is_copy));\n'
-        '  printf("%zu %zu %zu %zu %zu\\n", sizeof(tccl_pipeline_cfg), offsetof(tccl_pipeline_cfg, workgroups),\n'
+        '  printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(tccl_pipeline_cfg), offsetof(tccl_pipeline_cfg, workgroups),\n'
         '         offsetof(tccl_pipeline_cfg, lag), offsetof(tccl_pipeline_cfg, spin_limit),\n'
-        '         offsetof(tccl_pipeline_cfg, tile_kib));\n'
+        '         offsetof(tccl_pipeline_cfg, tile_kib), offsetof(tccl_pipeline_cfg, timeout_flag),\n'
+        '         offsetof(tccl_pipeline_cfg, flags));\n'
         '  printf("%d %d %d %d %d %d\\n", TCCL_ABI_VERSION, TCCL_MAX_WORLD, TCCL_MAX_JOBS, TCCL_BF16, TCCL_F32,\n'
         '         TCCL_CFG_PHASED);\n'
         '  return 0;\n}\n')
@@ -176,6 +179,7 @@ def test_struct_layouts_match_the_header(tmp_path):
     J = _lib.NodeJob
     assert job == [ctypes.sizeof(J), J.src.offset, J.dst.offset, J.numel.offset, J.is_copy.offset]
     P = _lib.PipelineCfg
-    assert pipe == [ctypes.sizeof(P), P.workgroups.offset, P.lag.offset, P.spin_limit.offset, P.tile_kib.offset]
+    assert pipe == [ctypes.sizeof(P), P.workgroups.offset, P.lag.offset, P.spin_limit.offset, P.tile_kib.offset,
+                    P.timeout_flag.offset, P.flags.offset]
     assert consts == [_lib.ABI_VERSION, _lib.MAX_WORLD, _lib.MAX_JOBS, _lib.TCCL_BF16, _lib.TCCL_F32,
                       _lib.CFG_PHASED]

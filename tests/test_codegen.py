@@ -63,6 +63,10 @@ def test_pipelined_kernel_uses_device_scope_accesses_and_no_cache_flushes(asm):
     two_shot = [b for n, b in bodies.items() if "two_shot_kernel" in n]
     assert len(tree) == 4 and len(two_shot) == 16
     for body in tree + two_shot:
+        # The place a workgroup draws at run time must reach the data path as a wave-uniform
+        # value: if it does not, every buffer access is wrapped in a loop over the distinct
+        # descriptors of the lanes (dozens of v_readfirstlane per access, +15 % run time).
+        assert body.count("v_readfirstlane_b32") < 64, "buffer descriptors are not wave-uniform"
         loads = re.findall(r"buffer_load_dwordx4[^\n]*", body)
         stores = re.findall(r"buffer_store_dwordx4[^\n]*", body)
         assert loads and stores

@@ -42,8 +42,15 @@ def upload(groups, bufs):
     return g
 
 
-def cfg(workgroups=0, lag=0, spin_limit=SPINS, tile_kib=0):
-    return _lib.PipelineCfg(workgroups, lag, spin_limit, tile_kib)
+def cfg(workgroups=0, lag=0, spin_limit=SPINS, tile_kib=0, draw=False):
+    """draw: the workgroups draw their places when they start to run (TCCL_PIPE_DRAW_PLACES)
+    instead of taking them from their hardware index."""
+    c = _lib.PipelineCfg(workgroups, lag, spin_limit, tile_kib)
+    c.flags = _lib.PIPE_DRAW_PLACES if draw else 0
+    return c
+
+
+BINDINGS = pytest.mark.parametrize("draw", [False, True], ids=["by-index", "drawn"])
 
 
 def pads_are_zero(group):
@@ -73,15 +80,16 @@ def run_and_check(group, want, what, **kw):
     (65_536 * 6 + 8 * 77, 0),       # whole 128 KiB chunks plus a ragged one
     (8 * 1_000_003, 65_536 * 3),    # chunks larger than a tile
 ])
-def test_pipelined_matches_oracle_and_schedule(world, maker, tile_kib, numel, chunk_elems, _gpu_hygiene, c_oracle):
+@BINDINGS
+def test_pipelined_matches_oracle_and_schedule(world, maker, tile_kib, numel, chunk_elems, draw, _gpu_hygiene, c_oracle):
     bufs = maker(world, numel, seed_base=900)
     want = torch_ref.double_tree_all_reduce(bufs)[0]
     if maker is seeded_randn:
         _, outs = c_oracle.double_tree_all_reduce_bf16([np_bits(b) for b in bufs])
         assert_bit_equal(from_np_bits(outs[0]), want, "oracles agree")
     g = upload(_gpu_hygiene, bufs)
-    got = run_and_check(g, want, f"W={world} n={numel} chunk={chunk_elems} tile={tile_kib}",
-                        chunk_elems=chunk_elems, pipeline_cfg=cfg(tile_kib=tile_kib))
+    got = run_and_check(g, want, f"W={world} n={numel} chunk={chunk_elems} tile={tile_kib} draw={draw}",
+                        chunk_elems=chunk_elems, pipeline_cfg=cfg(tile_kib=tile_kib, draw=draw))
     g2 = upload(_gpu_hygiene, bufs)
     levels = tccl_amd.double_tree_all_reduce_world(g2, fused=False, chunk_elems=chunk_elems)
     for r in range(world):
@@ -90,18 +98,20 @@ def test_pipelined_matches_oracle_and_schedule(world, maker, tile_kib, numel, ch
 
 @pytest.mark.parametrize("tile_kib", [32, 128])
 @pytest.mark.parametrize("workgroups,lag", [(8, 1), (8, 3), (16, 1), (64, 2), (256, 1), (256, 5), (0, 1), (0, 2), (0, 4)])
-def test_pipelined_grid_and_lag(workgroups, lag, tile_kib, _gpu_hygiene):
+@BINDINGS
+def test_pipelined_grid_and_lag(workgroups, lag, tile_kib, draw, _gpu_hygiene):
     """Any grid from one workgroup per rank upwards and any distance between the sweeps gives
     the same bits."""
     world, numel = 8, 65_536 * 40 + 4_096
     bufs = seeded_randn(world, numel, seed_base=910)
     want = torch_ref.double_tree_all_reduce(bufs)[0]
     g = upload(_gpu_hygiene, bufs)
-    run_and_check(g, want, f"wgs={workgroups} lag={lag} tile={tile_kib}",
-                  pipeline_cfg=cfg(workgroups, lag, tile_kib=tile_kib))
+    run_and_check(g, want, f"wgs={workgroups} lag={lag} tile={tile_kib} draw={draw}",
+                  pipeline_cfg=cfg(workgroups, lag, tile_kib=tile_kib, draw=draw))
 
 
-def test_pipelined_repeats_on_the_same_pads(_gpu_hygiene):
+@BINDINGS
+def test_pipelined_repeats_on_the_same_pads(draw, _gpu_hygiene):
     """The pads reset themselves: back-to-back collectives on one group, no clearing between."""
     world, numel = 8, 65_536 * 9
     g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
@@ -111,7 +121,7 @@ def test_pipelined_repeats_on_the_same_pads(_gpu_hygiene):
         for r, b in enumerate(bufs):
             g.tensor(r).copy_(b)
         want = torch_ref.double_tree_all_reduce(bufs)[0]
-        run_and_check(g, want, f"round {round_}", pipeline_cfg=cfg())
+        run_and_check(g, want, f"round {round_}", pipeline_cfg=cfg(draw=draw))
 
 
 def test_pipelined_fill_rank(_gpu_hygiene):
@@ -144,9 +154,12 @@ def test_pipelined_without_outputs_through_c_abi(_gpu_hygiene):
         assert_bit_equal(g.tensor(r), want, f"buffer {r}")
 
 
-def test_pipelined_full_size_properties(_gpu_hygiene):
-    """The full benchmark shape (8 x 256 MiB bf16, 128 KiB chunks): integer-valued inputs whose
-    sum is exact in every order, so the expected result is known without a CPU pass."""
+@BINDINGS
+def test_pipelined_full_size_properties(draw, _gpu_hygiene):
+    """The full benchmark shape as the baseline words it (8 x 256 MiB bf16, pipelined in 128 KiB
+    chunks = 65,536 elements, each worked as one 128 KiB tile): integer-valued inputs whose sum
+    is exact in every order, so the expected result is known without a CPU pass.  Then once more
+    with the library's own choice of chunk (32 KiB) on the same group."""
     world, numel = 8, 134_217_728
     g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
     _gpu_hygiene.append(g)
@@ -158,34 +171,69 @@ def test_pipelined_full_size_properties(_gpu_hygiene):
         total += vals.float()
     want = total.to(torch.bfloat16)       # |sum| <= 64: exact in bf16 at every node
     del total
-    outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1 << 20))
+    outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, chunk_elems=65_536,
+                                                 pipeline_cfg=cfg(spin_limit=1 << 20, tile_kib=128, draw=draw))
     assert tccl_amd.signal_pad_timeouts(g) == 0
     for r in range(world):
         assert torch.equal(outs[r], want), f"output {r}"
         assert torch.equal(g.tensor(r), want), f"buffer {r}"
     assert pads_are_zero(g)
+    # the buffers now all hold `want`: their all-reduce is 8 * want, still exact (|sum| <= 512)
+    outs = tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1 << 20, draw=draw))
+    assert tccl_amd.signal_pad_timeouts(g) == 0
+    want8 = (want.float() * 8).to(torch.bfloat16)
+    for r in range(world):
+        assert torch.equal(outs[r], want8), f"default chunks: output {r}"
+        assert torch.equal(g.tensor(r), want8), f"default chunks: buffer {r}"
+    assert pads_are_zero(g)
 
 
-def test_pipelined_expired_waits_drain_and_recover(_gpu_hygiene):
+@BINDINGS
+def test_pipelined_expired_waits_drain_and_recover(draw, _gpu_hygiene):
     """Failure handling, forced from the host: with a spin limit of one poll, waits expire (a
-    parent polls before its children can have finished a chunk).  The launch must still end,
-    report the time-outs, and the same group must work again once its pads are cleared."""
+    parent polls before its children can have finished a chunk).  The launch must still end
+    and count the time-outs, the next collective on the group must raise instead of working
+    on half-reduced buffers, and after that the group must work again."""
     world, numel = 8, 65_536 * 64
     bufs = seeded_randn(world, numel, seed_base=940)
     want = torch_ref.double_tree_all_reduce(bufs)[0]
     g = upload(_gpu_hygiene, bufs)
     print("pipelined: spin limit 1", flush=True)
-    tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1))
+    tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1, draw=draw))
     torch.cuda.synchronize()                         # the grid drained
     expired = tccl_amd.signal_pad_timeouts(g)
     if expired == 0:                                 # every signal happened to be there already
         for r in range(world):
             assert_bit_equal(g.tensor(r), want, f"buffer {r}")
         return
-    g.clear_signal_pads()
+    assert g.timeout_flag[0] == 1, "the kernel did not raise the host flag"
+    with pytest.raises(tccl_amd.TcclError) as err:
+        tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(draw=draw))
+    assert err.value.code == _lib.TCCL_ETIMEOUT
+    assert g.timeout_flag[0] == 0 and pads_are_zero(g), "raising must leave the group usable"
     for r, b in enumerate(bufs):
         g.tensor(r).copy_(b)
-    run_and_check(g, want, "after clearing the pads", pipeline_cfg=cfg())
+    run_and_check(g, want, "after the error", pipeline_cfg=cfg(draw=draw))
+
+
+def test_expired_wait_surfaces_at_the_next_collective_of_any_kind(_gpu_hygiene):
+    """The per-rank wrappers never hand out results of a group whose last signalling launch
+    timed out without saying so: whichever collective comes next raises (nobody has to know
+    about signal_pad_timeouts), exactly once."""
+    world, numel = 8, 65_536 * 64
+    bufs = seeded_randn(world, numel, seed_base=945)
+    g = upload(_gpu_hygiene, bufs)
+    print("pipelined through the per-rank wrapper: spin limit 1", flush=True)
+    tccl_amd.double_tree_all_reduce_world(g, pipelined=True, pipeline_cfg=cfg(spin_limit=1))
+    torch.cuda.synchronize()
+    if g.timeout_flag[0] == 0:
+        pytest.skip("no wait happened to expire in this run")
+    with pytest.raises(tccl_amd.TcclError, match="wait expired"):
+        tccl_amd.one_shot_all_reduce(g.tensor(0))
+    for r, b in enumerate(bufs):
+        g.tensor(r).copy_(b)
+    got = tccl_amd.one_shot_all_reduce(g.tensor(0))          # the error is reported once
+    assert_bit_equal(got, torch_ref.all_reduce(bufs), "one-shot after the error")
 
 
 def test_pipelined_argument_checks(_gpu_hygiene):
@@ -229,7 +277,8 @@ def two_shot_and_check(group, want, what, **kw):
 @pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("maker", [seeded_randn, seeded_uniform], ids=["bf16", "f32"])
 @pytest.mark.parametrize("vecs_per_share", [1, 3, 1_023, 1_024, 1_025, 70_001])
-def test_two_shot_one_launch_matches_oracle(world, maker, vecs_per_share, _gpu_hygiene, c_oracle):
+@BINDINGS
+def test_two_shot_one_launch_matches_oracle(world, maker, vecs_per_share, draw, _gpu_hygiene, c_oracle):
     """Every buffer and every output equals the one-shot all-reduce of the oracle, bit for
     bit: shares of one vector, around one 16 KiB tile (1,024 vectors) and many ragged tiles."""
     per_vec = 8 if maker is seeded_randn else 4
@@ -237,20 +286,21 @@ def test_two_shot_one_launch_matches_oracle(world, maker, vecs_per_share, _gpu_h
     bufs = maker(world, numel, seed_base=950)
     want = oracle_sum(c_oracle, bufs)
     g = upload(_gpu_hygiene, bufs)
-    two_shot_and_check(g, want, f"W={world} n={numel}", pipeline_cfg=cfg())
+    two_shot_and_check(g, want, f"W={world} n={numel} draw={draw}", pipeline_cfg=cfg(draw=draw))
     one = tccl_amd.one_shot_all_reduce(upload(_gpu_hygiene, bufs).tensor(0))
     assert_bit_equal(one, want, "one-shot kernel agrees")
 
 
 @pytest.mark.parametrize("workgroups", [8, 16, 24, 64, 512, 0])
 @pytest.mark.parametrize("with_outputs", [True, False])
-def test_two_shot_grid_and_in_place_only(workgroups, with_outputs, _gpu_hygiene, c_oracle):
+@BINDINGS
+def test_two_shot_grid_and_in_place_only(workgroups, with_outputs, draw, _gpu_hygiene, c_oracle):
     world, numel = 8, 8 * 8 * 40_001
     bufs = seeded_randn(world, numel, seed_base=960)
     want = oracle_sum(c_oracle, bufs)
     g = upload(_gpu_hygiene, bufs)
-    two_shot_and_check(g, want, f"wgs={workgroups} outs={with_outputs}", with_outputs=with_outputs,
-                       pipeline_cfg=cfg(workgroups))
+    two_shot_and_check(g, want, f"wgs={workgroups} outs={with_outputs} draw={draw}", with_outputs=with_outputs,
+                       pipeline_cfg=cfg(workgroups, draw=draw))
 
 
 def test_two_shot_order_sensitive_and_repeats(_gpu_hygiene):
@@ -265,7 +315,8 @@ def test_two_shot_order_sensitive_and_repeats(_gpu_hygiene):
     two_shot_and_check(g, torch.full((numel,), 28.0, dtype=torch.float32), "fill(rank)", pipeline_cfg=cfg())
 
 
-def test_two_shot_full_size(_gpu_hygiene):
+@BINDINGS
+def test_two_shot_full_size(draw, _gpu_hygiene):
     """The headline shape, 8 x 64 MiB bf16: against the one-shot kernel's result."""
     world, numel = 8, 33_554_432
     g = tccl_amd.empty_world(world, numel, torch.bfloat16, DEV)
@@ -274,7 +325,7 @@ def test_two_shot_full_size(_gpu_hygiene):
     for r in range(world):
         g.tensor(r).copy_(torch.randn(numel, generator=gen, device=DEV, dtype=torch.float32))
     want = tccl_amd.one_shot_all_reduce(g.tensor(0))
-    outs = tccl_amd.two_shot_all_reduce_world(g, pipeline_cfg=cfg(spin_limit=1 << 20))
+    outs = tccl_amd.two_shot_all_reduce_world(g, pipeline_cfg=cfg(spin_limit=1 << 20, draw=draw))
     assert tccl_amd.signal_pad_timeouts(g) == 0
     for r in range(world):
         assert torch.equal(outs[r].view(torch.int16), want.view(torch.int16)), f"output {r}"
@@ -282,25 +333,29 @@ def test_two_shot_full_size(_gpu_hygiene):
     assert pads_are_zero(g)
 
 
-def test_two_shot_expired_barrier_drains_and_recovers(_gpu_hygiene, c_oracle):
+@BINDINGS
+def test_two_shot_expired_barrier_drains_and_recovers(draw, _gpu_hygiene, c_oracle):
     """Failure handling, forced from the host: with one poll per wait the barrier expires
-    unless every peer happens to be there already; the launch ends either way, and after
-    clearing the pads the group works again."""
+    unless every peer happens to be there already; the launch ends either way, the next
+    collective raises, and then the group works again."""
     world, numel = 8, 8 * 8 * 200_000
     bufs = seeded_randn(world, numel, seed_base=970)
     want = oracle_sum(c_oracle, bufs)
     g = upload(_gpu_hygiene, bufs)
     print("two-shot: spin limit 1", flush=True)
-    tccl_amd.two_shot_all_reduce_world(g, pipeline_cfg=cfg(spin_limit=1))
+    tccl_amd.two_shot_all_reduce_world(g, pipeline_cfg=cfg(spin_limit=1, draw=draw))
     torch.cuda.synchronize()
     if tccl_amd.signal_pad_timeouts(g) == 0:
         for r in range(world):
             assert_bit_equal(g.tensor(r), want, f"buffer {r}")
         return
-    g.clear_signal_pads()
+    assert g.timeout_flag[0] == 1, "the kernel did not raise the host flag"
+    with pytest.raises(tccl_amd.TcclError) as err:
+        tccl_amd.two_shot_all_reduce_world(g, pipeline_cfg=cfg())
+    assert err.value.code == _lib.TCCL_ETIMEOUT
     for r, b in enumerate(bufs):
         g.tensor(r).copy_(b)
-    two_shot_and_check(g, want, "after clearing the pads", pipeline_cfg=cfg())
+    two_shot_and_check(g, want, "after the error", pipeline_cfg=cfg())
 
 
 def test_two_shot_argument_checks(_gpu_hygiene):

@@ -143,6 +143,7 @@ def test_random_signalling_kernels(case, c_oracle):
     i, tree_world, flat_world, dtype, numel, chunk_elems, pcfgd = case
     print(f"signalling case {i}: {case[1:]}", flush=True)
     pcfg = _lib.PipelineCfg(spin_limit=1 << 18, **pcfgd)
+    pcfg.flags = _lib.PIPE_DRAW_PLACES if i % 2 else 0          # both ways of binding places to workgroups
     # pipelined double tree
     bufs = _inputs(tree_world, numel, dtype, 3000 + i)
     want = torch_ref.double_tree_all_reduce(bufs)[0]
