@@ -50,6 +50,7 @@ enum {
     TCCL_EINVAL = -1,      /* NULL pointer, world/rank/dtype out of range, size mismatch */
     TCCL_EALIGN = -2,      /* a pointer or a row size is not a multiple of 16 bytes */
     TCCL_EPOW2 = -3,       /* tree world size is not a power of two >= 2 */
+    TCCL_ESCRATCH = -4,    /* the request needs more scratch memory than the library's static buffer holds */
     TCCL_ETIMEOUT = -5,    /* a wait of a signalling kernel expired (reported by host wrappers, never by a launch) */
     TCCL_EHIP_BASE = -1000 /* -(1000 + hipError_t) */
 };
@@ -275,6 +276,25 @@ int tccl_signal_pad_timeouts(const void *pad0, size_t pad_bytes, unsigned *timeo
 int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *signal_pads,
                              size_t pad_bytes, int world, size_t numel, int dtype,
                              const tccl_pipeline_cfg *cfg, void *stream);
+
+/* tccl_two_shot_all_reduce() for callers that cannot allocate the signal pads it needs -- code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same operation, same results, same cfg; the signal pads live
+ * in a static device array inside the library (TCCL_STATIC_SCRATCH_BYTES per GPU, held from
+ * the moment the library is loaded until the process ends), and the call allocates nothing on
+ * the device or the host: it enqueues one small kernel that clears the pads and then the
+ * all-reduce itself.  Limits: world <= TCCL_MAX_WORLD and at most TCCL_STATIC_MAX_WORKGROUPS
+ * workgroups per rank; a cfg->workgroups beyond world * TCCL_STATIC_MAX_WORKGROUPS is refused
+ * with TCCL_ESCRATCH (numel itself is not limited: the pads hold one flag per workgroup and
+ * peer, whatever the size).  Every call on a GPU uses that GPU's one array: calls that overlap
+ * in time on one GPU (two streams, two threads, two replaying graphs) race and must be kept
+ * apart by the caller; calls of one process outside graph capture are chained by the library
+ * like every signalling launch.  Time-outs are reported through cfg->timeout_flag only. */
+#define TCCL_STATIC_MAX_WORKGROUPS 1024
+#define TCCL_STATIC_SCRATCH_BYTES \
+    ((TCCL_STATIC_MAX_WORKGROUPS * TCCL_MAX_WORLD + TCCL_PAD_CONTROL_WORDS) * 4 * TCCL_MAX_WORLD)
+int tccl_two_shot_all_reduce_static(void *const *bufs, void *const *outs, int world, size_t numel, int dtype,
+                                    const tccl_pipeline_cfg *cfg, void *stream);
 
 /* A word for tccl_pipeline_cfg.timeout_flag: 32 bits of pinned, device-visible host memory,
  * zero to begin with.  The caller reads (and zeroes) it through the pointer.  Creating one

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtccl_amd.so")
 
 ABI_VERSION = 2
-TCCL_OK, TCCL_EINVAL, TCCL_EALIGN, TCCL_EPOW2, TCCL_ETIMEOUT = 0, -1, -2, -3, -5
+TCCL_OK, TCCL_EINVAL, TCCL_EALIGN, TCCL_EPOW2, TCCL_ESCRATCH, TCCL_ETIMEOUT = 0, -1, -2, -3, -4, -5
 MAX_WORLD = 8
 MAX_JOBS = 8
 
@@ -88,6 +88,7 @@ SIGNATURES = {
     "tccl_probe_write": (_I, [_P, _SZ, _P]),
     "tccl_signal_pad_timeouts": (_I, [_P, _SZ, ctypes.POINTER(ctypes.c_uint), _P]),
     "tccl_two_shot_all_reduce": (_I, [_PP, _PP, _PP, _SZ, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
+    "tccl_two_shot_all_reduce_static": (_I, [_PP, _PP, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
     "tccl_timeout_flag_create": (_I, [ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32))]),
     "tccl_timeout_flag_destroy": (_I, [ctypes.POINTER(ctypes.c_uint32)]),
     "tccl_double_tree_plan_create": (_I, [_PP, _PP, _I, _SZ, _I, _SZ, _PP]),

@@ -737,8 +737,30 @@ __global__ void __launch_bounds__(kPhasedBlock) two_shot_kernel(TwoShotArgs a)
     if (g != kNoPlace) two_shot_body<Sum, W>(a, rank, g, lds_ok);
 }
 
+// What the entry point without caller-owned pads asks for before its kernel: zero the first
+// flag_words words of each of `pads` pads of pad_words words starting at base, and the
+// control words.
+struct ClearRequest {
+    uint32_t *base;
+    uint32_t pad_words, flag_words;
+    int pads;
+};
+
+// Zeroes the first `flag_words` words of each of the gridDim.y pads and the control words at
+// the end of pad 0.  (A fill kernel, not a memset node: this entry point is meant to be
+// recorded into graphs.)
+__global__ void __launch_bounds__(kPhasedBlock) clear_pads_kernel(uint32_t *base, uint32_t pad_words, uint32_t flag_words)
+{
+    uint32_t *pad = base + static_cast<size_t>(blockIdx.y) * pad_words;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < flag_words; i += gridDim.x * blockDim.x)
+        __hip_atomic_store(pad + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (blockIdx.x == 0 && blockIdx.y == 0)
+        for (uint32_t i = threadIdx.x; i < kCtlWords; i += blockDim.x)
+            __hip_atomic_store(base + pad_words - kCtlWords + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <class Sum, int W>
-static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, hipStream_t s)
+static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, const ClearRequest *clear, hipStream_t s)
 {
     static std::once_flag once;
     static int resident = 0;
@@ -766,7 +788,14 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, hipS
         per_rank = workgroups_per_rank(tiles, most < fit ? most : fit);
     }
     a.wgs_per_rank = static_cast<int>(per_rank);
-    SignallingLaunch guard(s);
+    SignallingLaunch guard(s); // from here on the stream is behind the device's previous signalling kernel
+    if (clear != nullptr) {
+        const dim3 cgrid((clear->flag_words + kPhasedBlock * 4 - 1) / (kPhasedBlock * 4), clear->pads);
+        hipLaunchKernelGGL(clear_pads_kernel, cgrid, dim3(kPhasedBlock), 0, s, clear->base, clear->pad_words,
+                           clear->flag_words);
+        const hipError_t ce = hipGetLastError();
+        if (ce != hipSuccess) return hip_code(ce);
+    }
     hipLaunchKernelGGL((two_shot_kernel<Sum, W>), dim3(static_cast<unsigned>(per_rank * W)), dim3(kPhasedBlock), 0, s,
                        a);
     const hipError_t e = hipGetLastError();
@@ -775,17 +804,18 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, hipS
 }
 
 template <class Sum>
-static int launch_two_shot_world(const TwoShotArgs &a, int wgs_wanted, size_t pad_words, hipStream_t s)
+static int launch_two_shot_world(const TwoShotArgs &a, int wgs_wanted, size_t pad_words, const ClearRequest *clear,
+                                 hipStream_t s)
 {
     switch (a.world) {
-    case 1: return launch_two_shot<Sum, 1>(a, wgs_wanted, pad_words, s);
-    case 2: return launch_two_shot<Sum, 2>(a, wgs_wanted, pad_words, s);
-    case 3: return launch_two_shot<Sum, 3>(a, wgs_wanted, pad_words, s);
-    case 4: return launch_two_shot<Sum, 4>(a, wgs_wanted, pad_words, s);
-    case 5: return launch_two_shot<Sum, 5>(a, wgs_wanted, pad_words, s);
-    case 6: return launch_two_shot<Sum, 6>(a, wgs_wanted, pad_words, s);
-    case 7: return launch_two_shot<Sum, 7>(a, wgs_wanted, pad_words, s);
-    case 8: return launch_two_shot<Sum, 8>(a, wgs_wanted, pad_words, s);
+    case 1: return launch_two_shot<Sum, 1>(a, wgs_wanted, pad_words, clear, s);
+    case 2: return launch_two_shot<Sum, 2>(a, wgs_wanted, pad_words, clear, s);
+    case 3: return launch_two_shot<Sum, 3>(a, wgs_wanted, pad_words, clear, s);
+    case 4: return launch_two_shot<Sum, 4>(a, wgs_wanted, pad_words, clear, s);
+    case 5: return launch_two_shot<Sum, 5>(a, wgs_wanted, pad_words, clear, s);
+    case 6: return launch_two_shot<Sum, 6>(a, wgs_wanted, pad_words, clear, s);
+    case 7: return launch_two_shot<Sum, 7>(a, wgs_wanted, pad_words, clear, s);
+    case 8: return launch_two_shot<Sum, 8>(a, wgs_wanted, pad_words, clear, s);
     default: return TCCL_EINVAL;
     }
 }
@@ -809,7 +839,7 @@ static int two_shot_check(void *const *bufs, void *const *outs, int world, size_
 
 // The launch itself: `pads` are the W signal pads (device addresses), each of pad_bytes.
 static int two_shot_launch(void *const *bufs, void *const *outs, uint32_t *const *pads, size_t pad_bytes, int world,
-                           size_t numel, int dtype, const tccl_pipeline_cfg *cfg, hipStream_t s)
+                           size_t numel, int dtype, const tccl_pipeline_cfg *cfg, const ClearRequest *clear, hipStream_t s)
 {
     TwoShotArgs a = {};
     for (int r = 0; r < world; ++r) {
@@ -825,8 +855,8 @@ static int two_shot_launch(void *const *bufs, void *const *outs, uint32_t *const
     a.report = cfg ? cfg->timeout_flag : nullptr;
     a.draw = (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
     const int wgs = cfg ? cfg->workgroups : 0;
-    return dtype == TCCL_BF16 ? launch_two_shot_world<Bf16Sum>(a, wgs, pad_words, s)
-                              : launch_two_shot_world<F32Sum>(a, wgs, pad_words, s);
+    return dtype == TCCL_BF16 ? launch_two_shot_world<Bf16Sum>(a, wgs, pad_words, clear, s)
+                              : launch_two_shot_world<F32Sum>(a, wgs, pad_words, clear, s);
 }
 
 } // namespace tccl
@@ -848,7 +878,77 @@ extern "C" int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, vo
         pads[r] = static_cast<uint32_t *>(signal_pads[r]);
     }
     if (nothing) return TCCL_OK;
-    return two_shot_launch(bufs, outs, pads, pad_bytes, world, numel, dtype, cfg, static_cast<hipStream_t>(stream));
+    return two_shot_launch(bufs, outs, pads, pad_bytes, world, numel, dtype, cfg, nullptr,
+                           static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------------------------------ the entry point that allocates nothing
+namespace tccl {
+
+// Signal pads of the two-shot all-reduce for callers that cannot bring their own: W pads of
+// kStaticPadBytes each, side by side in one array that every GPU holds from the moment the
+// library is loaded until the process ends.  A pad has room for TCCL_STATIC_MAX_WORKGROUPS
+// workgroups per rank in a world of TCCL_MAX_WORLD, plus the control words.
+constexpr size_t kStaticPadBytes =
+    (static_cast<size_t>(TCCL_STATIC_MAX_WORKGROUPS) * TCCL_MAX_WORLD + kCtlWords) * sizeof(uint32_t);
+static_assert(kStaticPadBytes % 16 == 0, "pads must stay 16-byte aligned");
+static_assert(kStaticPadBytes * TCCL_MAX_WORLD == TCCL_STATIC_SCRATCH_BYTES, "header and library disagree");
+
+static __device__ __align__(256) unsigned char scratch[TCCL_STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device (every GPU has its own copy of the array
+// at its own address).  Looked up once per device; nullptr with *err set when that fails.
+static unsigned char *scratch_on_current_device(hipError_t *err)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex m;
+    static unsigned char *ptrs[kMaxDevices] = {};
+    int dev = 0;
+    *err = hipGetDevice(&dev);
+    if (*err != hipSuccess) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) {
+        *err = hipErrorInvalidDevice;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(m);
+    if (ptrs[dev] == nullptr) {
+        void *p = nullptr;
+        *err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (*err != hipSuccess || p == nullptr) {
+            if (*err == hipSuccess) *err = hipErrorInvalidSymbol;
+            return nullptr;
+        }
+        ptrs[dev] = static_cast<unsigned char *>(p);
+    }
+    return ptrs[dev];
+}
+
+} // namespace tccl
+
+extern "C" int tccl_two_shot_all_reduce_static(void *const *bufs, void *const *outs, int world, size_t numel,
+                                               int dtype, const tccl_pipeline_cfg *cfg, void *stream)
+{
+    bool nothing = false;
+    const int rc = two_shot_check(bufs, outs, world, numel, dtype, &nothing);
+    if (rc != TCCL_OK) return rc;
+    // more workgroups per rank than a static pad has flags for: say so instead of clamping
+    if (cfg != nullptr && cfg->workgroups > TCCL_STATIC_MAX_WORKGROUPS * world) return TCCL_ESCRATCH;
+    if (nothing) return TCCL_OK;
+    hipError_t e = hipSuccess;
+    unsigned char *base = scratch_on_current_device(&e);
+    if (base == nullptr) return hip_code(e);
+    uint32_t *pads[TCCL_MAX_WORLD];
+    for (int r = 0; r < world; ++r) pads[r] = reinterpret_cast<uint32_t *>(base + static_cast<size_t>(r) * kStaticPadBytes);
+    // The array keeps whatever the last call left: flags of a call whose waits expired would let
+    // this call's waits pass too early.  Clear what this call can touch, in stream order, behind
+    // the device's previous signalling kernel.
+    ClearRequest clear;
+    clear.base = reinterpret_cast<uint32_t *>(base);
+    clear.pad_words = static_cast<uint32_t>(kStaticPadBytes / sizeof(uint32_t));
+    clear.flag_words = static_cast<uint32_t>(TCCL_STATIC_MAX_WORKGROUPS) * world;
+    clear.pads = world;
+    return two_shot_launch(bufs, outs, pads, kStaticPadBytes, world, numel, dtype, cfg, &clear,
+                           static_cast<hipStream_t>(stream));
 }
 
 // A 32-bit word in pinned host memory that the GPU can write: a caller without HIP bindings

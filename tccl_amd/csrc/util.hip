@@ -97,6 +97,7 @@ extern "C" const char *tccl_error_string(int code)
     case TCCL_EINVAL: return "invalid argument (NULL pointer, world/rank/dtype out of range)";
     case TCCL_EALIGN: return "pointer or size is not a multiple of 16 bytes";
     case TCCL_EPOW2: return "world size is not a power of two >= 2";
+    case TCCL_ESCRATCH: return "the request needs more scratch memory than the library's static buffer holds";
     case TCCL_ETIMEOUT: return "a wait of a signalling kernel expired: that collective's results are incomplete";
     default:
         if (code <= TCCL_EHIP_BASE) return hipGetErrorString(static_cast<hipError_t>(TCCL_EHIP_BASE - code));

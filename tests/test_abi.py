@@ -110,6 +110,13 @@ def test_argument_checks_return_codes_without_launching():
     assert two(good, None, pads, 4090, 2, 64, 0, None, None) == -1            # pad size not a multiple of 16
     assert two(null, None, pads, 4096, 2, 64, 0, None, None) == -1
     assert two(good, None, pads, 4096, 2, 0, 0, None, None) == 0
+    static = lib.tccl_two_shot_all_reduce_static
+    assert static(good, None, 0, 64, 0, None, None) == -1
+    assert static(good, None, 9, 64, 0, None, None) == -1
+    assert static(good, None, 2, 24, 0, None, None) == -2
+    assert static(null, None, 2, 64, 0, None, None) == -1
+    assert static(good, None, 2, 64, 0, ctypes.byref(_lib.PipelineCfg(2 * 1024 + 1, 0, 0, 0)), None) == _lib.TCCL_ESCRATCH
+    assert static(good, None, 2, 0, 0, None, None) == 0
     assert lib.tccl_timeout_flag_create(None) == -1 and lib.tccl_timeout_flag_destroy(None) == -1
     assert lib.tccl_probe_read(good, 2, 64, None, None) == -1
     assert lib.tccl_probe_read(good, 9, 64, out, None) == -1
