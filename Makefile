@@ -15,11 +15,11 @@ test: build oracle  ## everything that needs no GPU
 test-gpu:         ## bit-exact parity on an MI355X (library must be built)
 	$(PYTHON) -m pytest tests -x -q -m gpu
 
-bench:            ## one JSON line: W=8 x 64 MiB bf16 all-reduce
+bench:            ## one JSON line: W=8 x 64 MiB bf16 all-reduce, the other ops and the size sweep
 	$(PYTHON) bench.py
 
-sweep:            ## every operation and size, JSON lines on stderr
-	$(PYTHON) bench.py --sweep
+sweep:            ## one operation alone, e.g. make sweep OP=reduce_scatter_bf16
+	$(PYTHON) bench.py --only $(OP)
 
 clean:
 	rm -rf tccl_amd/csrc/_obj tccl_amd/libtccl_amd.so tests/c_client/build

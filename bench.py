@@ -4,17 +4,27 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Workload (the one the headline metric is quoted on): one-shot all-reduce (sum) over W=8
-virtual-rank buffers of 64 MiB bf16 each (33,554,432 elements ~N(0,1), seeded per rank),
-all resident in HBM before the timed region.  A step is one call of
-``tccl_amd.one_shot_all_reduce`` (output allocation from torch's caching allocator plus one
-kernel launch through the C ABI).  Prints ONE JSON line on stdout.
+virtual-rank buffers of 64 MiB bf16 each (33,554,432 elements, buffer r made on the CPU by
+``torch.manual_seed(r); torch.randn(n, dtype=bfloat16)``), all resident in HBM before the
+timed region.  A step is one call of ``tccl_amd.one_shot_all_reduce`` (output allocation from
+torch's caching allocator plus one kernel launch through the C ABI).  Prints ONE JSON line on
+stdout.
 
 Algorithmic bytes per step: (W + 1) * N * 2 = 603,979,776 (W*N read, N written).
+
+Besides the headline the line carries: the same step rotated over 8 buffer sets (nothing
+served from the 256 MB memory-side cache), the memory system's own read-pass and write-pass
+times, latencies at 1 MiB (single launch, launch floor, graph replay), the torch CPU oracle
+timed on the host, every other operation of the path at its benchmark shape (cold), and a
+compact size sweep.  ``--only OP`` runs one operation alone, for profiler runs whose kernel
+statistics must hold one kernel at one size.
 """
 from __future__ import annotations
 
 import argparse
 import ctypes
+import gc
+import hashlib
 import json
 import os
 import statistics
@@ -29,32 +39,39 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 WORLD = 8
 BYTES_PER_BUF = 64 << 20
 LAT_BYTES_PER_BUF = 1 << 20
+COLD_BYTES = 1 << 30            # a rotation touches at least this much between two uses of a byte (cache: 256 MB)
+MIN_SETS = 4                    # ... over at least this many disjoint buffer sets
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "headline_traffic.json")
 
-# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs of this script
-# (FETCH_SIZE 262,354.07 KiB and WRITE_SIZE 65,536.00 KiB per dispatch), each scaled by what
-# the same counter reads for the 256 MiB plain copy of --calibrate-copy (factors 1.99959 and
-# 0.99996): 524,600 KiB fetched + 65,533 KiB written.
-MEASURED_TRAFFIC_BYTES = 604_296_372
+ONLY_OPS = ["all_reduce", "all_reduce_rotated", "probe_read", "probe_write", "reduce_scatter_bf16", "reduce_scatter_f32",
+            "all_gather_bf16", "all_gather_f32", "all_gather_int8", "tree_reduce_c0", "tree_reduce_c1",
+            "tree_reduce_c2", "tree_copy_1", "tree_copy_2", "double_tree_level", "double_tree_pipelined",
+            "double_tree_pipelined_drawn", "two_shot", "two_shot_drawn", "copy_calibration", "placement", "ceilings"]
 
 
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
-    p.add_argument("--warmup", type=int, default=150,
-                   help="untimed steps first; 150 (13 ms) because launches 30-100 after idle run 1-2 %% slower "
-                        "than the steady state while the clocks settle")
+    p.add_argument("--warmup", type=int, default=20, help="untimed steps right before the timed ones")
+    p.add_argument("--preheat", type=int, default=300,
+                   help="launches of the headline step before the warm-up, reported as preheat_launches: "
+                        "the first 100 or so launches after an idle period run 1-2 %% slower while the clocks settle, "
+                        "so a short --warmup would time the ramp")
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     p.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU work budget for the baseline leg")
     p.add_argument("--no-other-ops", action="store_true",
-                   help="skip the short timings of reduce-scatter, all-gather and the tree node steps")
+                   help="skip reduce-scatter, all-gather, the tree node steps and the signalling kernels")
+    p.add_argument("--no-sweep", action="store_true", help="skip the size sweep")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run 20 plain copies of 256 MiB (tccl_tree_copy_step), so that a rocprofv3 --pmc "
                         "run of this command holds a kernel of known traffic to scale the counters by")
-    p.add_argument("--sweep", action="store_true",
-                   help="also time every op and size of the sweep; written to stderr as JSON lines")
+    p.add_argument("--only", choices=ONLY_OPS,
+                   help="run this one operation alone (--steps launches after --warmup) and print a small JSON line")
     return p.parse_args()
 
+
+# ------------------------------------------------------------------------------------------ timing helpers
 
 class HipEvents:
     """HIP events from the library, recorded on the stream the kernels are launched on."""
@@ -81,21 +98,13 @@ class HipEvents:
             self.lib.tccl_event_destroy(e)
 
 
-def make_world(tccl_amd, torch, world, numel, dtype, device):
-    group = tccl_amd.empty_world(world, numel, dtype, device)
-    for r in range(world):
-        gen = torch.Generator(device=device)
-        gen.manual_seed(r)
-        if dtype == torch.int8:
-            group.tensor(r).copy_(torch.randint(-128, 128, (numel,), dtype=dtype, device=device, generator=gen))
-        else:
-            group.tensor(r).copy_(torch.randn(numel, dtype=torch.float32, device=device, generator=gen))
-    return group
+def raw_stream(torch):
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
 def time_steps(torch, lib, fn, steps, warmup):
     """(wall ms per step, HIP-event ms per step) over exactly `steps` calls."""
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    stream = raw_stream(torch)
     ev = HipEvents(lib, 2)
     for _ in range(warmup):
         fn()
@@ -113,8 +122,8 @@ def time_steps(torch, lib, fn, steps, warmup):
 
 
 def latency_p50_us(torch, lib, fn, reps=300, warmup=30):
-    """Median over single-launch HIP-event pairs."""
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """Median (and 99th percentile) over single-launch HIP-event pairs."""
+    stream = raw_stream(torch)
     ev = HipEvents(lib, 2 * reps)
     for _ in range(warmup):
         fn()
@@ -128,6 +137,79 @@ def latency_p50_us(torch, lib, fn, reps=300, warmup=30):
     ev.close()
     return statistics.median(us), us[int(0.99 * (reps - 1))]
 
+
+def free(torch):
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+class Rotation:
+    """Calls fn(k) for k = 0, 1, ..., nsets-1, 0, ...: one launch per call, each on its own set of
+    buffers, so that `nsets` x bytes_per_set (>= COLD_BYTES) lie between two uses of a byte."""
+
+    def __init__(self, fn, nsets):
+        self.fn, self.nsets, self.turn = fn, nsets, 0
+
+    def __call__(self):
+        self.turn += 1
+        return self.fn(self.turn % self.nsets)
+
+
+def sets_for(bytes_per_set):
+    return max(MIN_SETS, -(-COLD_BYTES // bytes_per_set))
+
+
+# ------------------------------------------------------------------------------------------ inputs
+
+def cpu_recipe(torch, world, numel, dtype):
+    """The baseline's input recipe: buffer r = manual_seed(r); randn(n, dtype) made on the CPU."""
+    out = []
+    for r in range(world):
+        torch.manual_seed(r)
+        out.append(torch.randn(numel, dtype=dtype))
+    return out
+
+
+class Noise:
+    """One block of device-made N(0,1) values (seeded) from which timing-only buffers are filled:
+    values do not matter to a streaming kernel's time, and making 20 GB of them would."""
+
+    def __init__(self, torch, device, nbytes=256 << 20):
+        gen = torch.Generator(device=device)
+        gen.manual_seed(1234)
+        self.torch = torch
+        self.f32 = torch.randn(nbytes // 4, dtype=torch.float32, device=device, generator=gen)
+        self.bf16 = self.f32[: nbytes // 8].to(torch.bfloat16)     # nbytes/4 bytes of bf16
+
+    def fill(self, t, salt=0):
+        """t <- noise of t's dtype (int8: the raw bytes), starting at a salt-dependent offset."""
+        torch = self.torch
+        if t.dtype == torch.bfloat16:
+            src = self.bf16
+        elif t.dtype == torch.float32:
+            src = self.f32
+        else:
+            src = self.f32.view(torch.int8)
+        n, m = t.numel(), src.numel()
+        flat = t.view(-1)
+        off = (salt * 4099 * 8) % max(1, m // 2)
+        done = 0
+        while done < n:
+            take = min(n - done, m - off)
+            flat[done:done + take].copy_(src[off:off + take])
+            done += take
+            off = 0
+        return t
+
+
+def make_world(tccl_amd, torch, noise, world, numel, dtype, device, salt=0):
+    group = tccl_amd.empty_world(world, numel, dtype, device)
+    for r in range(world):
+        noise.fill(group.tensor(r), salt + r)
+    return group
+
+
+# ------------------------------------------------------------------------------------------ CPU baseline
 
 def cpu_baseline(torch, bufs_cpu, seconds):
     """The torch CPU oracle on the same workload, all host cores torch will use."""
@@ -143,6 +225,340 @@ def cpu_baseline(torch, bufs_cpu, seconds):
     return statistics.median(times), len(times)
 
 
+# ------------------------------------------------------------------------------------------ single operations
+
+class Ops:
+    """Every operation of the path at its benchmark shape, each as (callable doing ONE launch on
+    rotated buffers, algorithmic bytes per launch, kernel it launches)."""
+
+    def __init__(self, torch, tccl_amd, lib, plib, noise, device):
+        self.torch, self.tccl_amd, self.lib, self.plib, self.noise, self.device = torch, tccl_amd, lib, plib, noise, device
+        self.keep = []
+
+    def close(self):
+        for g in self.keep:
+            if hasattr(g, "world_size"):
+                self.tccl_amd.unregister(g)
+        self.keep = []
+        free(self.torch)
+
+    def _worlds(self, nsets, world, numel, dtype):
+        gs = [make_world(self.tccl_amd, self.torch, self.noise, world, numel, dtype, self.device, salt=17 * k)
+              for k in range(nsets)]
+        self.keep += gs
+        return gs
+
+    def all_reduce(self, rotated):
+        torch, numel = self.torch, BYTES_PER_BUF // 2
+        nbytes = (WORLD + 1) * BYTES_PER_BUF
+        nsets = sets_for(nbytes) if rotated else 1
+        nsets = max(nsets, 8) if rotated else 1
+        gs = self._worlds(nsets, WORLD, numel, torch.bfloat16)
+        outs = [torch.empty_like(g.tensor(0)) for g in gs]
+        fn = Rotation(lambda k: self.tccl_amd.one_shot_all_reduce(gs[k].tensor(0), out=outs[k]), nsets)
+        return fn, nbytes, "sum_phased_kernel<Bf16Sum, 8, 1, true>"
+
+    def probe_read(self):
+        torch = self.torch
+        gs = self._worlds(1, WORLD, BYTES_PER_BUF // 2, torch.bfloat16)
+        sink = torch.zeros(4096, dtype=torch.uint8, device=self.device)
+        s = raw_stream(torch)
+        fn = lambda: self.plib.tccl_probe_read(gs[0].ptr_array, WORLD, BYTES_PER_BUF, sink.data_ptr(), s)
+        self.keep.append(sink)
+        return fn, WORLD * BYTES_PER_BUF, "probe_read_kernel<8>"
+
+    def probe_write(self):
+        torch = self.torch
+        out = torch.empty(BYTES_PER_BUF, dtype=torch.uint8, device=self.device)
+        s = raw_stream(torch)
+        self.keep.append(out)
+        return (lambda: self.plib.tccl_probe_write(out.data_ptr(), BYTES_PER_BUF, s)), BYTES_PER_BUF, "probe_write_kernel"
+
+    def reduce_scatter(self, dtype):
+        """W=8 inputs of 67,108,864 elements, rank 3's share (the baseline's shape); two input sets
+        alternate and the share is written to rotating outputs: 2 x 8 x 16 MiB of input shares
+        (bf16) cannot be held by the cache together with everything else that is touched."""
+        torch, numel = self.torch, 67_108_864
+        esize = 2 if dtype == torch.bfloat16 else 4
+        per = numel // WORLD
+        nbytes = (WORLD + 1) * per * esize
+        nsets = sets_for(nbytes)
+        gs = self._worlds(nsets, WORLD, numel, dtype)
+        outs = [torch.empty(per, dtype=dtype, device=self.device) for _ in range(nsets)]
+        fn = Rotation(lambda k: self.tccl_amd.reduce_scatter(gs[k].tensor(3), out=outs[k]), nsets)
+        return fn, nbytes, "sum_phased_kernel<%s, 8, ...>" % ("Bf16Sum" if esize == 2 else "F32Sum")
+
+    def all_gather(self, dtype):
+        torch, numel = self.torch, 8_388_608
+        esize = torch.empty(0, dtype=dtype).element_size()
+        nbytes = 2 * WORLD * numel * esize
+        nsets = sets_for(nbytes)
+        gs = self._worlds(nsets, WORLD, numel, dtype)
+        outs = [torch.empty((WORLD, numel), dtype=dtype, device=self.device) for _ in range(nsets)]
+        fn = Rotation(lambda k: self.tccl_amd.all_gather(gs[k].tensor(0), WORLD, out=outs[k]), nsets)
+        return fn, nbytes, "pack_kernel"
+
+    def tree_step(self, children=None, destinations=None):
+        """One node step on a 128 MiB half in 128 KiB chunks through the level launcher: a reduce
+        step (own + `children` child buffers, in place) or a copy step (parent -> `destinations`)."""
+        from tccl_amd import _lib
+        torch, half = self.torch, 67_108_864
+        nbuf = (children + 1) if children is not None else (destinations + 1)
+        nbytes = ((children + 2) if children is not None else (1 + destinations)) * half * 2
+        nsets = sets_for(nbuf * half * 2)
+        jobs = []
+        for k in range(nsets):
+            bufs = [self.noise.fill(torch.empty(half, dtype=torch.bfloat16, device=self.device), 31 * k + i)
+                    for i in range(nbuf)]
+            self.keep += bufs
+            j = (_lib.NodeJob * 1)()
+            if children is not None:
+                kids = [bufs[1].data_ptr() if children >= 1 else None, bufs[2].data_ptr() if children >= 2 else None]
+                j[0].src[0], j[0].src[1], j[0].src[2] = kids[0], kids[1], bufs[0].data_ptr()
+                j[0].dst[0], j[0].dst[1] = bufs[0].data_ptr(), None
+                j[0].numel, j[0].is_copy = half, 0
+            else:
+                j[0].src[0], j[0].src[1], j[0].src[2] = bufs[0].data_ptr(), None, None
+                j[0].dst[0], j[0].dst[1] = bufs[1].data_ptr(), bufs[2].data_ptr() if destinations == 2 else None
+                j[0].numel, j[0].is_copy = half, 1
+            jobs.append(j)
+        s = raw_stream(torch)
+        fn = Rotation(lambda k: self.lib.tccl_tree_level(jobs[k], 1, 0, 65_536, s), nsets)
+        return fn, nbytes, "tree_level_kernel / tree_copy_level_kernel"
+
+    def double_tree(self, how):
+        """Whole double-tree all-reduce, W=8 x 256 MiB (4 GiB touched per call)."""
+        torch = self.torch
+        gs = self._worlds(1, WORLD, 134_217_728, torch.bfloat16)
+        g = gs[0]
+        t = self.tccl_amd
+        if how == "level":
+            fn = lambda: t.double_tree_all_reduce_world(g, fused=False, pipelined=False)
+        elif how == "pipelined_128k":
+            fn = lambda: t.double_tree_all_reduce_world(g, pipelined=True, chunk_elems=65_536)
+        else:
+            fn = lambda: t.double_tree_all_reduce_world(g, pipelined=True, draw_places=(how == "pipelined_drawn"))
+        return fn, 74 * (128 << 20), "tree_level_kernel x 6 / tree_pipelined_kernel", g
+
+    def two_shot(self, drawn=False):
+        torch = self.torch
+        gs = self._worlds(1, WORLD, BYTES_PER_BUF // 2, torch.bfloat16)
+        g = gs[0]
+        fn = lambda: self.tccl_amd.two_shot_all_reduce_world(g, with_outputs=False, draw_places=drawn)
+        return fn, (3 * WORLD - 1) * BYTES_PER_BUF, "two_shot_kernel<Bf16Sum, 8>", g
+
+    def copy_calibration(self):
+        torch, nbytes = self.torch, 256 << 20
+        src = torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device=self.device)
+        dst = torch.empty_like(src)
+        s = raw_stream(torch)
+        self.keep += [src, dst]
+        return (lambda: self.lib.tccl_tree_copy_step(src.data_ptr(), dst.data_ptr(), None, nbytes, s)), 2 * nbytes, "copy_kernel"
+
+    def get(self, name):
+        torch = self.torch
+        if name == "all_reduce":
+            return self.all_reduce(False)
+        if name == "all_reduce_rotated":
+            return self.all_reduce(True)
+        if name in ("probe_read", "probe_write", "copy_calibration"):
+            return getattr(self, name)()
+        if name.startswith("reduce_scatter_"):
+            return self.reduce_scatter(torch.bfloat16 if name.endswith("bf16") else torch.float32)
+        if name.startswith("all_gather_"):
+            return self.all_gather({"bf16": torch.bfloat16, "f32": torch.float32, "int8": torch.int8}[name[11:]])
+        if name.startswith("tree_reduce_c"):
+            return self.tree_step(children=int(name[-1]))
+        if name.startswith("tree_copy_"):
+            return self.tree_step(destinations=int(name[-1]))
+        if name == "double_tree_level":
+            return self.double_tree("level")[:3]
+        if name == "double_tree_pipelined":
+            return self.double_tree("pipelined")[:3]
+        if name == "double_tree_pipelined_drawn":
+            return self.double_tree("pipelined_drawn")[:3]
+        if name in ("two_shot", "two_shot_drawn"):
+            return self.two_shot(name.endswith("drawn"))[:3]
+        raise ValueError(name)
+
+
+def cold_ceilings(torch, lib, plib, device):
+    """What the memory system gives the simplest kernels on data that is in no cache (4 GiB arena,
+    every launch on the next 512 MiB of it): the reference points for the operations' own rates."""
+    arena = torch.empty(4 << 30, dtype=torch.uint8, device=device)
+    arena.view(torch.int32).fill_(0x3C003C00)
+    sink = torch.zeros(4096, dtype=torch.uint8, device=device)
+    s = raw_stream(torch)
+    base = arena.data_ptr()
+    R = 512 << 20
+    out = {}
+    _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_read_dense(base + k * R, R, sink.data_ptr(), s), 8), 32, 16)
+    out["read_dense_gbs"] = round(R / (ms * 1e-3) / 1e9, 1)
+    ptrs = [(ctypes.c_void_p * 8)(*[base + k * R + i * (64 << 20) for i in range(8)]) for k in range(8)]
+    _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_read(ptrs[k], 8, 64 << 20, sink.data_ptr(), s), 8), 32, 16)
+    out["read_8_streams_128KiB_tiles_gbs"] = round(R / (ms * 1e-3) / 1e9, 1)
+    W = 64 << 20
+    _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_write(base + k * W, W, s), 64), 128, 64)
+    out["write_64MiB_128KiB_tiles_gbs"] = round(W / (ms * 1e-3) / 1e9, 1)
+    C = 128 << 20
+    _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_copy(base + (2 * k) * C, base + (2 * k + 1) * C, C, s), 16), 32, 16)
+    out["copy_128MiB_gbs"] = round(2 * C / (ms * 1e-3) / 1e9, 1)
+    out["note"] = "benchlib/probe.hip kernels on a 4 GiB arena, every launch on the next part of it (nothing cached)"
+    del arena
+    free(torch)
+    return out
+
+
+def run_only(args, torch, tccl_amd, lib, plib, device):
+    if args.only == "placement":
+        return placement(torch, plib, device)
+    if args.only == "ceilings":
+        print(json.dumps({"only": "ceilings", **cold_ceilings(torch, lib, plib, device)}), flush=True)
+        return
+    noise = Noise(torch, device)
+    ops = Ops(torch, tccl_amd, lib, plib, noise, device)
+    fn, nbytes, kernel = ops.get(args.only)
+    _, ms = time_steps(torch, lib, fn, args.steps, args.warmup)
+    line = {"only": args.only, "kernel": kernel, "steps": args.steps, "warmup": args.warmup,
+            "avg_launch_us": round(ms * 1e3, 2), "algorithmic_bytes": nbytes,
+            "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_8TBs": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    ops.close()
+    if args.calibrate_copy:
+        calibrate_copy(torch, lib, device)
+    print(json.dumps(line), flush=True)
+
+
+def calibrate_copy(torch, lib, device):
+    nbytes = 256 << 20
+    src = torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device=device)
+    dst = torch.empty_like(src)
+    stream = raw_stream(torch)
+    for _ in range(20):
+        assert lib.tccl_tree_copy_step(src.data_ptr(), dst.data_ptr(), None, nbytes, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+
+
+def placement(torch, plib, device):
+    """Where the hardware puts the workgroups of grids of 4 and 6 per compute unit."""
+    for n in (1024, 1536):
+        where = torch.full((2 * n,), -1, dtype=torch.int32, device=device)
+        assert plib.tccl_probe_placement(where.data_ptr(), n, 20000, raw_stream(torch)) == 0
+        torch.cuda.synchronize()
+        w = where.cpu().view(n, 2)
+        hw, xcc = w[:, 0], w[:, 1] & 15
+        b = torch.arange(n)
+        print(f"grid {n}: workgroups on XCD (index mod 8): {int((xcc == b % 8).sum())} of {n}")
+        cu = (xcc << 16) | (hw & 0xFF00)
+        per = torch.unique(cu, return_counts=True)[1]
+        print(f"grid {n}: distinct compute units {per.numel()}, workgroups per unit min {int(per.min())} max {int(per.max())}")
+        if n == 1024:
+            for x in (0, 1):
+                seq = [int(v) for v in hw[x::8][:64]]
+                print(f"XCD {x}, i-th workgroup -> se.cu:", " ".join(f"{(v >> 13) & 7}.{(v >> 8) & 15}" for v in seq))
+
+
+# ------------------------------------------------------------------------------------------ sweep
+
+def sweep(torch, tccl_amd, lib, noise, device):
+    """The all-reduce size sweep of the baseline (W in {2,4,8}, 16 KiB .. 256 MiB per buffer in
+    powers of 4) through the C entry point on separate allocations: p50 us of single launches
+    up to 1 MiB, GB/s on algorithmic bytes from 4 MiB, rotated over enough buffer sets (at least
+    MIN_SETS) that COLD_BYTES lie between two uses of a byte.  Also the CPU-runnable shape (W=8 x 8 MiB), cold."""
+    out = {"note": "all-reduce, bf16, C entry point; p50_us: single launches on one buffer set; "
+                   "cold_gbs: algorithmic bytes / mean launch time, rotated over `sets` buffer sets (>= 4 sets and >= 1 GiB "
+                   "touched between two uses of a byte)"}
+    stream = raw_stream(torch)
+    sizes = [16 << 10 << (2 * i) for i in range(8)]
+
+    def one(world, nbytes, steps):
+        numel = nbytes // 2
+        touched = (world + 1) * nbytes
+        nsets = 1 if nbytes <= (1 << 20) else sets_for(touched)
+        sets = []
+        for k in range(nsets):
+            bufs = [noise.fill(torch.empty(numel, dtype=torch.bfloat16, device=device), 13 * k + r) for r in range(world)]
+            o = torch.empty(numel, dtype=torch.bfloat16, device=device)
+            sets.append((bufs, o, ctypes.cast((ctypes.c_void_p * world)(*[b.data_ptr() for b in bufs]),
+                                               ctypes.POINTER(ctypes.c_void_p))))
+        fn = Rotation(lambda k: lib.tccl_all_reduce_sum(sets[k][2], world, sets[k][1].data_ptr(), numel, 0, stream), nsets)
+        if nsets == 1:
+            p50, _ = latency_p50_us(torch, lib, fn, reps=100, warmup=10)
+            res = {"p50_us": round(p50, 2)}
+        else:
+            _, ms = time_steps(torch, lib, fn, steps, max(3, nsets // 4))
+            res = {"cold_gbs": round(touched / (ms * 1e-3) / 1e9, 1), "us": round(ms * 1e3, 2), "sets": nsets}
+        del sets
+        return res
+
+    for world in (2, 4, 8):
+        row = {}
+        for nbytes in sizes:
+            label = f"{nbytes >> 10}KiB" if nbytes < (1 << 20) else f"{nbytes >> 20}MiB"
+            row[label] = one(world, nbytes, 24 if nbytes <= (16 << 20) else 12)
+            free(torch)
+        out[f"w{world}"] = row
+    out["config1_w8_8MiB_cold"] = one(8, 8 << 20, 36)
+    free(torch)
+    return out
+
+
+# ------------------------------------------------------------------------------------------ other ops
+
+def other_ops(torch, tccl_amd, lib, plib, noise, device):
+    """The other operations of the path at their full benchmark shapes: GB/s on algorithmic bytes
+    from HIP events (30 launches after 6 warm-ups), every one rotated over enough disjoint buffers
+    that nothing is served from the 256 MB memory-side cache."""
+    out = {}
+    ops = Ops(torch, tccl_amd, lib, plib, noise, device)
+    for name in ("reduce_scatter_bf16", "reduce_scatter_f32", "all_gather_bf16", "all_gather_f32", "all_gather_int8",
+                 "tree_reduce_c0", "tree_reduce_c1", "tree_reduce_c2", "tree_copy_1", "tree_copy_2"):
+        fn, nbytes, _ = ops.get(name)
+        _, ms = time_steps(torch, lib, fn, 30, 6)
+        out[name] = {"gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "us": round(ms * 1e3, 2),
+                     "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 3)}
+        ops.close()
+    # whole double-tree all-reduce, W=8 x 256 MiB: level schedule, pipelined single launch (both chunk sizes, both bindings)
+    for how, key in (("level", "double_tree_w8_256MiB_level_schedule_ms"),
+                     ("pipelined_128k", "double_tree_w8_256MiB_pipelined_128KiB_chunks_ms"),
+                     ("pipelined", "double_tree_w8_256MiB_pipelined_32KiB_chunks_ms"),
+                     ("pipelined_drawn", "double_tree_w8_256MiB_pipelined_drawn_places_ms")):
+        fn, nbytes, _, g = ops.double_tree(how)
+        _, ms = time_steps(torch, lib, fn, 5, 2)
+        out[key] = round(ms, 3)
+        out["double_tree_pipelined_expired_waits"] = out.get("double_tree_pipelined_expired_waits", 0) + \
+            tccl_amd.signal_pad_timeouts(g)
+        ops.close()
+    for drawn, key in ((False, "two_shot_in_place_all_ranks_w8_64MiB_us"), (True, "two_shot_drawn_places_us")):
+        fn, nbytes, _, g = ops.two_shot(drawn)
+        _, ms = time_steps(torch, lib, fn, 20, 5)
+        out[key] = round(ms * 1e3, 1)
+        out["two_shot_expired_waits"] = out.get("two_shot_expired_waits", 0) + tccl_amd.signal_pad_timeouts(g)
+        ops.close()
+    return out
+
+
+# ------------------------------------------------------------------------------------------ traffic evidence
+
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel from the committed counter summary, and
+    whether the kernel's sources are still the ones it was measured on."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, "profiles/headline_traffic.json missing", None
+    h = hashlib.sha256()
+    for rel in rec.get("sources", []):
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    same = h.hexdigest()[:16] == rec.get("sources_sha256_16")
+    return rec["traffic_bytes"], "profiles/headline_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, " \
+        f"scaled by a 256 MiB copy: x{rec['fetch_scale']} / x{rec['write_scale']})", same
+
+
+# ------------------------------------------------------------------------------------------ main
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -152,19 +568,30 @@ def main():
 
     import torch
     import tccl_amd
+    from benchlib import probe
     lib = tccl_amd.load_library()
+    plib = probe.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device = "cuda:0"
     torch.cuda.set_device(0)
 
+    if args.only:
+        return run_only(args, torch, tccl_amd, lib, plib, device)
+
     numel = BYTES_PER_BUF // 2
-    group = make_world(tccl_amd, torch, WORLD, numel, torch.bfloat16, device)
+    bufs_cpu = cpu_recipe(torch, WORLD, numel, torch.bfloat16)
+    group = tccl_amd.empty_world(WORLD, numel, torch.bfloat16, device)
+    for r in range(WORLD):
+        group.tensor(r).copy_(bufs_cpu[r])
     mine = group.tensor(0)
     algo_bytes = (WORLD + 1) * numel * 2
+    noise = Noise(torch, device)
 
     def step():
         return tccl_amd.one_shot_all_reduce(mine)
 
+    for _ in range(args.preheat):
+        step()
     wall_ms, dev_ms = time_steps(torch, lib, step, args.steps, args.warmup)
     gbs_wall = algo_bytes / (wall_ms * 1e-3) / 1e9
     gbs_dev = algo_bytes / (dev_ms * 1e-3) / 1e9
@@ -175,19 +602,15 @@ def main():
     # and serves a little of the input; rotated like this every byte really moves over HBM.
     rot_ms = None
     try:
-        extra = [make_world(tccl_amd, torch, WORLD, numel, torch.bfloat16, device) for _ in range(7)]
+        extra = [make_world(tccl_amd, torch, noise, WORLD, numel, torch.bfloat16, device, salt=100 * k) for k in range(7)]
         firsts = [mine] + [g.tensor(0) for g in extra]
         outs = [torch.empty_like(mine) for _ in range(8)]
-        turn = [0]
-
-        def rotated_step():
-            turn[0] += 1
-            return tccl_amd.one_shot_all_reduce(firsts[turn[0] % 8], out=outs[turn[0] % 8])
-
-        _, rot_ms = time_steps(torch, lib, rotated_step, args.steps, args.warmup)
+        rotated_step = Rotation(lambda k: tccl_amd.one_shot_all_reduce(firsts[k], out=outs[k]), 8)
+        _, rot_ms = time_steps(torch, lib, rotated_step, max(args.steps, 40), max(args.warmup, 16))
         for g in extra:
             tccl_amd.unregister(g)
-        del extra, firsts, outs
+        del extra, firsts, outs, rotated_step
+        free(torch)
     except RuntimeError as e:            # e.g. not enough free memory for seven more sets
         print(f"rotated measurement skipped: {e}", file=sys.stderr)
 
@@ -196,30 +619,51 @@ def main():
     # is a read phase followed by a write burst, so their total is its practical bound here.
     sink = torch.zeros(4096, dtype=torch.uint8, device=device)
     probe_out = torch.empty_like(mine)
-    pstream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    _, read_ms = time_steps(torch, lib, lambda: lib.tccl_probe_read(group.ptr_array, WORLD, BYTES_PER_BUF,
-                                                                    sink.data_ptr(), pstream), 100, 50)
-    _, write_ms = time_steps(torch, lib, lambda: lib.tccl_probe_write(probe_out.data_ptr(), BYTES_PER_BUF, pstream),
+    pstream = raw_stream(torch)
+    _, read_ms = time_steps(torch, lib, lambda: plib.tccl_probe_read(group.ptr_array, WORLD, BYTES_PER_BUF,
+                                                                     sink.data_ptr(), pstream), 100, 50)
+    _, write_ms = time_steps(torch, lib, lambda: plib.tccl_probe_write(probe_out.data_ptr(), BYTES_PER_BUF, pstream),
                              100, 50)
     ceilings = {
         "read_8x64MiB_us": round(read_ms * 1e3, 2), "read_gbs": round(WORLD * BYTES_PER_BUF / (read_ms * 1e-3) / 1e9, 1),
         "write_64MiB_us": round(write_ms * 1e3, 2), "write_gbs": round(BYTES_PER_BUF / (write_ms * 1e-3) / 1e9, 1),
         "read_pass_plus_write_pass_us": round((read_ms + write_ms) * 1e3, 2),
         "sum_kernel_us": round(dev_ms * 1e3, 2),
-        "note": "tccl_probe_read / tccl_probe_write: the read half and the write half of the sum kernel on their "
-                "own, same buffers and launch shape, 100 launches each",
+        "note": "the read half and the write half of the sum kernel on their own (benchlib/probe.hip), same buffers "
+                "and launch shape, 100 launches each on one buffer set",
     }
     del probe_out
 
-    # p50 latency at 1 MiB per buffer: prefix views of the same allocations
+    # latency at 1 MiB per buffer: prefix views of the same allocations
     lat_numel = LAT_BYTES_PER_BUF // 2
     small = mine[:lat_numel]
     p50_us, p99_us = latency_p50_us(torch, lib, lambda: tccl_amd.one_shot_all_reduce(small))
     # the same launch through the C entry point alone (output allocated once, no wrapper work)
     small_out = torch.empty_like(small)
-    raw_stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    c_call = lambda: lib.tccl_all_reduce_sum(group.ptr_array, WORLD, small_out.data_ptr(), lat_numel, 0, raw_stream)
+    c_call = lambda: lib.tccl_all_reduce_sum(group.ptr_array, WORLD, small_out.data_ptr(), lat_numel, 0, pstream)
     p50_c_us, _ = latency_p50_us(torch, lib, c_call)
+    # what an empty kernel costs under the same event bracketing: the floor of this measurement
+    floor_us, _ = latency_p50_us(torch, lib, lambda: plib.tccl_probe_empty(pstream))
+    # the C entry point recorded into a HIP graph and replayed: what a caller that removes the launch path pays
+    graph_us = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            lib.tccl_all_reduce_sum(group.ptr_array, WORLD, small_out.data_ptr(), lat_numel, 0, raw_stream(torch))
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            assert lib.tccl_all_reduce_sum(group.ptr_array, WORLD, small_out.data_ptr(), lat_numel, 0, raw_stream(torch)) == 0
+        graph_us, _ = latency_p50_us(torch, lib, graph.replay)
+        # ten replays back to back, per replay
+        _, g10 = time_steps(torch, lib, graph.replay, 500, 50)
+        graph_b2b_us = g10 * 1e3
+        del graph
+    except RuntimeError as e:
+        print(f"graph replay measurement skipped: {e}", file=sys.stderr)
+        graph_b2b_us = None
     # and what one wrapper call costs end to end when calls are issued back to back
     back_wall_ms, back_dev_ms = time_steps(torch, lib, lambda: tccl_amd.one_shot_all_reduce(small), 500, 50)
 
@@ -228,6 +672,7 @@ def main():
     bus = ctypes.c_int()
     l2 = ctypes.c_size_t()
     lib.tccl_device_info(ctypes.byref(cu), ctypes.byref(clk), ctypes.byref(bus), ctypes.byref(l2))
+    traffic, traffic_source, traffic_current = measured_traffic()
 
     result = {
         "metric": "achieved HBM GB/s (% of 8 TB/s) W=8 bf16 reduce @64MiB/buf; p50 us @1MiB",
@@ -236,23 +681,29 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "preheat_launches": args.preheat,
         "ms_per_step": round(wall_ms, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",                      # the sums are accumulated in fp32 ...
         "io_dtype": "bf16",                  # ... over bf16 inputs, rounded once to a bf16 output
-        "data": "synthetic N(0,1), seeded per virtual rank, resident in HBM",
+        "data": "synthetic: buffer r = torch.manual_seed(r); torch.randn(n, dtype=bfloat16) on the CPU, copied to its own "
+                "HBM allocation before the timed region (rotated sets, other ops and the sweep: device-made N(0,1))",
         "config": {"workload": "one-shot all-reduce sum, W=8 virtual ranks, 64 MiB bf16 per buffer "
                                "(33,554,432 elements), one MI355X",
                    "world": WORLD, "bytes_per_buffer": BYTES_PER_BUF, "algorithmic_bytes_per_step": algo_bytes},
         "pct_of_peak": round(100.0 * gbs_wall / HBM_PEAK_GBS, 2),
         "rotated_over_8_buffer_sets": None if rot_ms is None else {
-            "gbs": round(algo_bytes / (rot_ms * 1e-3) / 1e9, 1), "avg_launch_us": round(rot_ms * 1e3, 2)},
+            "gbs": round(algo_bytes / (rot_ms * 1e-3) / 1e9, 1), "avg_launch_us": round(rot_ms * 1e3, 2),
+            "frac": round(algo_bytes / (rot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "memory_system_ceilings": ceilings,
         "p50_us_at_1MiB": round(p50_us, 2),
         "p99_us_at_1MiB": round(p99_us, 2),
         "p50_us_at_1MiB_c_entry_point_only": round(p50_c_us, 2),
+        "launch_floor_us": round(floor_us, 2),
+        "p50_us_at_1MiB_graph_replay": None if graph_us is None else round(graph_us, 2),
+        "us_per_replay_at_1MiB_graph_back_to_back": None if graph_b2b_us is None else round(graph_b2b_us, 2),
         "us_per_call_at_1MiB_back_to_back": round(back_dev_ms * 1e3, 2),
         "roofline": {
             "bound": "hbm",
@@ -260,7 +711,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs_dev / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
+            "traffic_measured_on_these_sources": traffic_current,
             "kernel": "tccl::sum_phased_kernel<Bf16Sum, 8, 1, true>",
             "avg_launch_us": round(dev_ms * 1e3, 2),
             "algorithmic_bytes": algo_bytes,
@@ -270,7 +723,6 @@ def main():
     }
 
     if not args.no_cpu_baseline:
-        bufs_cpu = [group.tensor(r).cpu() for r in range(WORLD)]
         med_s, nruns = cpu_baseline(torch, bufs_cpu, args.cpu_seconds)
         # the GPU result must equal the CPU oracle's on the very same inputs
         from oracle import torch_ref
@@ -300,221 +752,33 @@ def main():
             "one_thread": {"value": round(algo_bytes / one_s / 1e9, 2), "unit": "GB/s",
                            "ms_per_pass": round(one_s * 1e3, 1)},
             "cpu_model": model, "torch_version": torch.__version__})
-        del bufs_cpu
+    del bufs_cpu
+
+    tccl_amd.unregister(group)
+    del group, mine, small, small_out
+    free(torch)
+
+    try:
+        result["cold_memory_ceilings"] = cold_ceilings(torch, lib, plib, device)
+    except RuntimeError as e:
+        result["cold_memory_ceilings"] = {"error": str(e)[:200]}
 
     if not args.no_other_ops:
         try:
-            result["other_ops"] = other_ops(torch, tccl_amd, lib, device)
+            result["other_ops"] = other_ops(torch, tccl_amd, lib, plib, noise, device)
         except RuntimeError as e:        # the headline must still be printed
             result["other_ops"] = {"error": str(e)[:200]}
 
-    if args.calibrate_copy:
-        nbytes = 256 << 20
-        src = torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device=device)
-        dst = torch.empty_like(src)
-        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        for _ in range(20):
-            assert lib.tccl_tree_copy_step(src.data_ptr(), dst.data_ptr(), None, nbytes, stream) == 0
-        torch.cuda.synchronize()
-        assert torch.equal(src, dst)
-        del src, dst
+    if not args.no_sweep:
+        try:
+            result["sweep"] = sweep(torch, tccl_amd, lib, noise, device)
+        except RuntimeError as e:
+            result["sweep"] = {"error": str(e)[:200]}
 
-    if args.sweep:
-        run_sweep(torch, tccl_amd, lib, device)
+    if args.calibrate_copy:
+        calibrate_copy(torch, lib, device)
 
     print(json.dumps(result), flush=True)
-
-
-def other_ops(torch, tccl_amd, lib, device):
-    """The other operations of the path at their full benchmark shapes, bf16: GB/s on algorithmic
-    bytes from HIP events (30 launches after 5 warm-ups).  Each rotates over enough disjoint
-    buffers that nothing is served from the 256 MB memory-side cache."""
-    import gc
-    from tccl_amd import _lib
-    out = {}
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-
-    # reduce-scatter: W=8 inputs of 67,108,864 elements, every rank's share in turn (8 x 144 MiB touched)
-    g = make_world(tccl_amd, torch, 8, 67_108_864, torch.bfloat16, device)
-    turn = [0]
-
-    def rs():
-        turn[0] += 1
-        return tccl_amd.reduce_scatter(g.tensor(turn[0] % 8))
-    _, ms = time_steps(torch, lib, rs, 32, 8)
-    out["reduce_scatter_w8_64Mi_el_gbs"] = round(9 * (67_108_864 // 8) * 2 / (ms * 1e-3) / 1e9, 1)
-    tccl_amd.unregister(g)
-    del g
-    gc.collect()
-    torch.cuda.empty_cache()
-
-    # all-gather: W=8 x 8,388,608 elements, two groups alternating (2 x 256 MiB touched)
-    gs = [make_world(tccl_amd, torch, 8, 8_388_608, torch.bfloat16, device) for _ in range(2)]
-
-    def ag():
-        turn[0] += 1
-        return tccl_amd.all_gather(gs[turn[0] % 2].tensor(0), 8)
-    _, ms = time_steps(torch, lib, ag, 30, 6)
-    out["all_gather_w8_8Mi_el_gbs"] = round(2 * 8 * 8_388_608 * 2 / (ms * 1e-3) / 1e9, 1)
-    for g in gs:
-        tccl_amd.unregister(g)
-    del gs
-    gc.collect()
-    torch.cuda.empty_cache()
-
-    # tree node steps on 128 MiB halves in 128 KiB chunks: four different jobs in turn (2 GiB touched)
-    half = 67_108_864
-    bufs = [torch.randn(half, dtype=torch.float32, device=device).to(torch.bfloat16) for _ in range(12)]
-    jobs = [(_lib.NodeJob * 1)() for _ in range(4)]
-
-    def set_reduce():
-        for i, j in enumerate(jobs):
-            j[0].src[0], j[0].src[1], j[0].src[2] = bufs[3 * i + 1].data_ptr(), bufs[3 * i + 2].data_ptr(), bufs[3 * i].data_ptr()
-            j[0].dst[0], j[0].dst[1] = bufs[3 * i].data_ptr(), None
-            j[0].numel, j[0].is_copy = half, 0
-
-    def set_copy():
-        for i, j in enumerate(jobs):
-            j[0].src[0], j[0].src[1], j[0].src[2] = bufs[3 * i].data_ptr(), None, None
-            j[0].dst[0], j[0].dst[1] = bufs[3 * i + 1].data_ptr(), bufs[3 * i + 2].data_ptr()
-            j[0].numel, j[0].is_copy = half, 1
-
-    def level():
-        turn[0] += 1
-        return lib.tccl_tree_level(jobs[turn[0] % 4], 1, 0, 65_536, stream)
-    set_reduce()
-    _, ms = time_steps(torch, lib, level, 32, 8)
-    out["tree_reduce_step_2_children_128MiB_gbs"] = round(4 * half * 2 / (ms * 1e-3) / 1e9, 1)
-    set_copy()
-    _, ms = time_steps(torch, lib, level, 32, 8)
-    out["tree_copy_step_2_destinations_128MiB_gbs"] = round(3 * half * 2 / (ms * 1e-3) / 1e9, 1)
-    del bufs
-    gc.collect()
-    torch.cuda.empty_cache()
-
-    # whole double-tree all-reduce, W=8 x 256 MiB in 128 KiB chunks (4 GiB touched per call): the level
-    # schedule (one launch per tree level) and the pipelined single launch (ranks signal each other per chunk)
-    g = make_world(tccl_amd, torch, 8, 134_217_728, torch.bfloat16, device)
-    _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, fused=False, pipelined=False), 5, 2)
-    out["double_tree_w8_256MiB_level_schedule_ms"] = round(ms, 3)
-    _, ms = time_steps(torch, lib,
-                       lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True, chunk_elems=65_536), 5, 2)
-    out["double_tree_w8_256MiB_pipelined_128KiB_chunks_ms"] = round(ms, 3)
-    _, ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, pipelined=True), 5, 2)
-    out["double_tree_w8_256MiB_pipelined_32KiB_chunks_ms"] = round(ms, 3)
-    out["double_tree_pipelined_expired_waits"] = tccl_amd.signal_pad_timeouts(g)
-    tccl_amd.unregister(g)
-    del g
-    gc.collect()
-    torch.cuda.empty_cache()
-
-    # all W ranks' all-reduce in place in one launch (two-shot with the blockwise barrier), 8 x 64 MiB
-    g = make_world(tccl_amd, torch, 8, 33_554_432, torch.bfloat16, device)
-    _, ms = time_steps(torch, lib, lambda: tccl_amd.two_shot_all_reduce_world(g, with_outputs=False), 20, 5)
-    out["two_shot_in_place_all_ranks_w8_64MiB_us"] = round(ms * 1e3, 1)
-    out["two_shot_expired_waits"] = tccl_amd.signal_pad_timeouts(g)
-    tccl_amd.unregister(g)
-    del g
-    gc.collect()
-    torch.cuda.empty_cache()
-    return out
-
-
-def run_sweep(torch, tccl_amd, lib, device):
-    """Every op at its full benchmark shape and the all-reduce size sweep; JSON lines on
-    stderr (GB/s on algorithmic bytes from HIP events; p50 us per launch)."""
-    import gc
-
-    def emit(**kw):
-        print(json.dumps(kw), file=sys.stderr, flush=True)
-
-    def rate(fn, nbytes, steps=50, warmup=10):
-        _, dev_ms = time_steps(torch, lib, fn, steps, warmup)
-        return round(nbytes / (dev_ms * 1e-3) / 1e9, 1), round(dev_ms * 1e3, 2)
-
-    def drop(g):
-        tccl_amd.unregister(g)
-        gc.collect()
-        torch.cuda.empty_cache()
-
-    # all-reduce sweep: W in {2,4,8}, 16 KiB .. 256 MiB per buffer in powers of 4
-    for world in (2, 4, 8):
-        g = make_world(tccl_amd, torch, world, (256 << 20) // 2, torch.bfloat16, device)
-        nbytes = 16 << 10
-        while nbytes <= (256 << 20):
-            view = g.tensor(0)[:nbytes // 2]
-            fn = lambda: tccl_amd.one_shot_all_reduce(view)
-            gbs, us = rate(fn, (world + 1) * nbytes)
-            p50, _ = latency_p50_us(torch, lib, fn, reps=200, warmup=10)
-            emit(op="all_reduce", world=world, dtype="bf16", bytes_per_buffer=nbytes, gbs=gbs, avg_us=us,
-                 p50_us=round(p50, 2))
-            nbytes *= 4
-        drop(g)
-
-    # reduce-scatter, rank 3 of 8, 67,108,864 elements per input
-    for dtype, name in ((torch.bfloat16, "bf16"), (torch.float32, "f32")):
-        g = make_world(tccl_amd, torch, 8, 67_108_864, dtype, device)
-        t = g.tensor(3)
-        per_bytes = t.numel() // 8 * t.element_size()
-        gbs, us = rate(lambda: tccl_amd.reduce_scatter(t), 9 * per_bytes)
-        emit(op="reduce_scatter", world=8, rank=3, dtype=name, numel=t.numel(), gbs=gbs, avg_us=us)
-        drop(g)
-
-    # all-gather pack, 8 x 8,388,608 elements
-    for dtype, name in ((torch.bfloat16, "bf16"), (torch.float32, "f32"), (torch.int8, "int8")):
-        g = make_world(tccl_amd, torch, 8, 8_388_608, dtype, device)
-        t = g.tensor(0)
-        gbs, us = rate(lambda: tccl_amd.all_gather(t, 8), 2 * 8 * t.numel() * t.element_size())
-        emit(op="all_gather", world=8, dtype=name, numel=t.numel(), gbs=gbs, avg_us=us)
-        drop(g)
-
-    # double-tree node step on one 128 MiB half in 128 KiB chunks: reduce (own + 2 children,
-    # in place) and forward copy (parent -> own + output), via the level launcher
-    from tccl_amd import _lib
-    half = 67_108_864
-    bufs = [torch.randn(half, dtype=torch.float32, device=device).to(torch.bfloat16) for _ in range(5)]
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    job = (_lib.NodeJob * 1)()
-    for c in (0, 1, 2):
-        kids = [bufs[1].data_ptr() if c >= 1 else None, bufs[2].data_ptr() if c >= 2 else None]
-        job[0].src[0], job[0].src[1], job[0].src[2] = kids[0], kids[1], bufs[0].data_ptr()
-        job[0].dst[0], job[0].dst[1] = bufs[0].data_ptr(), None
-        job[0].numel, job[0].is_copy = half, 0
-        gbs, us = rate(lambda: lib.tccl_tree_level(job, 1, 0, 65_536, stream), (c + 2) * half * 2)
-        emit(op="tree_reduce_step", children=c, chunk_bytes=131072, bytes_per_half=half * 2, gbs=gbs, avg_us=us)
-    for ndst in (1, 2):
-        job[0].src[0], job[0].src[1], job[0].src[2] = bufs[0].data_ptr(), None, None
-        job[0].dst[0], job[0].dst[1] = bufs[3].data_ptr(), bufs[4].data_ptr() if ndst == 2 else None
-        job[0].numel, job[0].is_copy = half, 1
-        gbs, us = rate(lambda: lib.tccl_tree_level(job, 1, 0, 65_536, stream), (1 + ndst) * half * 2)
-        emit(op="tree_copy_step", destinations=ndst, chunk_bytes=131072, bytes_per_half=half * 2, gbs=gbs, avg_us=us)
-    del bufs
-    gc.collect()
-    torch.cuda.empty_cache()
-
-    # whole double-tree all-reduce, W=8 x 256 MiB
-    g = make_world(tccl_amd, torch, 8, 134_217_728, torch.bfloat16, device)
-    _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(g, fused=False, pipelined=False), 5, 2)
-    emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20, schedule="one launch per tree level",
-         ms=round(dev_ms, 3))
-    for chunk_kib in (128, 32):
-        _, dev_ms = time_steps(torch, lib, lambda: tccl_amd.double_tree_all_reduce_world(
-            g, pipelined=True, chunk_elems=chunk_kib * 512), 5, 2)
-        emit(op="double_tree_all_reduce", world=8, bytes_per_buffer=256 << 20,
-             schedule=f"one persistent launch, ranks signal each other per {chunk_kib} KiB chunk",
-             ms=round(dev_ms, 3), expired_waits=tccl_amd.signal_pad_timeouts(g))
-    drop(g)
-
-    # every rank's all-reduce in one launch (two-shot with the blockwise barrier), W=8 x 64 MiB
-    g = make_world(tccl_amd, torch, 8, 33_554_432, torch.bfloat16, device)
-    for with_outputs in (False, True):
-        _, dev_ms = time_steps(torch, lib,
-                               lambda: tccl_amd.two_shot_all_reduce_world(g, with_outputs=with_outputs), 20, 5)
-        nbytes = ((3 if not with_outputs else 4) * 8 - 1) * 33_554_432 * 2
-        emit(op="two_shot_all_reduce_all_ranks", world=8, bytes_per_buffer=64 << 20, outputs=with_outputs,
-             avg_us=round(dev_ms * 1e3, 1), gbs=round(nbytes / (dev_ms * 1e-3) / 1e9, 1),
-             expired_waits=tccl_amd.signal_pad_timeouts(g))
-    drop(g)
 
 
 if __name__ == "__main__":

@@ -1,0 +1,37 @@
+/*
+ * probe.h -- measuring kernels used by bench.py only (benchlib/libtccl_probe.so).  Not part of
+ * the product library or its ABI; none of them has a counterpart in the reference.
+ */
+#ifndef TCCL_PROBE_H
+#define TCCL_PROBE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The read half of the large all-reduce on its own: reads and reduces `world` buffers of
+ * bytes_per_buffer each (bf16 arithmetic, the sum kernel's launch shape) and stores nothing
+ * (`sink`: 4,096 bytes of device memory that receives a checksum in one case out of 2^32,
+ * which is what keeps the loads alive). */
+int tccl_probe_read(const void *const *bufs, int world, size_t bytes_per_buffer, void *sink, void *stream);
+/* The write half: fills `bytes` at dst with a pattern, 32 stores per lane back to back. */
+int tccl_probe_write(void *dst, size_t bytes, void *stream);
+/* One contiguous range read front to back by the whole GPU (grid-stride, streaming loads): the
+ * fastest way found to read HBM, the reference point for every read rate in the benchmark. */
+int tccl_probe_read_dense(const void *buf, size_t bytes, void *sink, void *stream);
+/* A plain copy in the launch shape that is fastest on uncached data: the reference point for the
+ * copies (all-gather, tree copy step). */
+int tccl_probe_copy(const void *src, void *dst, size_t bytes, void *stream);
+/* One empty kernel: what a timed single launch costs when the kernel does nothing. */
+int tccl_probe_empty(void *stream);
+/* out[2*b] = HW_REG_HW_ID, out[2*b+1] = HW_REG_XCC_ID of workgroup b of a grid of `workgroups`
+ * x 256 lanes, each holding its slot for hold_us microseconds. */
+int tccl_probe_placement(uint32_t *out, int workgroups, int hold_us, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -98,8 +98,9 @@ int tccl_all_reduce_sum_ex(const void *const *bufs, int world, void *out, size_t
 /* One rank's share of a reduce-scatter: out[j] = sum_i bufs[i][rank*P + j],
  * P = numel_total / world, j < P.
  * Replaces one_shot_reduce_scatter_kernel, triton_reduce_scatter.py:59-92 (launched at
- * :116-126).  rank*P*esize must be a multiple of 16 (the reference requires
- * numel % (8*world) == 0, :101-104). */
+ * :116-126).  numel_total must be a multiple of world and P*esize a multiple of 16 (the
+ * reference requires numel % (8*world) == 0, :101-104); TCCL_EALIGN otherwise, for every rank
+ * alike. */
 int tccl_reduce_scatter_sum(const void *const *bufs, int world, int rank, void *out,
                             size_t numel_total, int dtype, void *stream);
 int tccl_reduce_scatter_sum_ex(const void *const *bufs, int world, int rank, void *out,
@@ -312,19 +313,6 @@ int tccl_event_record(void *event, void *stream);
 int tccl_event_synchronize(void *event);
 int tccl_event_elapsed_ms(void *start, void *stop, float *ms_out);
 int tccl_stream_synchronize(void *stream);
-
-/* Measuring kernels: the read half and the write half of the large all-reduce on their
- * own, with its launch shape (256 lanes, 128 KiB tiles, two workgroups per compute unit, one
- * launch per resident wave of tiles).  The large sum is a read phase followed by a write
- * burst, so "time of tccl_probe_read + time of tccl_probe_write" is the bound the memory
- * system sets for it on the GPU at hand; a benchmark prints it beside the sum's own time.
- * tccl_probe_read reads and reduces `world` buffers of bytes_per_buffer each (bf16
- * arithmetic) and stores nothing (`sink`: 4,096 bytes of device memory that receives a
- * checksum in one case out of 2^32, which is what keeps the loads alive);
- * tccl_probe_write fills `bytes` at dst with a pattern.  No counterpart in the reference. */
-int tccl_probe_read(const void *const *bufs, int world, size_t bytes_per_buffer, void *sink,
-                    void *stream);
-int tccl_probe_write(void *dst, size_t bytes, void *stream);
 
 /* Device facts used for reporting: compute units, memory clock (kHz), bus width (bits),
  * L2 bytes.  Any pointer may be NULL. */

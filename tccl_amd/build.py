@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "_obj")
 LIB_PATH = os.path.join(HERE, "libtccl_amd.so")
 
-SOURCES = ["sum.hip", "gather.hip", "tree.hip", "pipeline.hip", "probe.hip", "util.hip"]
+SOURCES = ["sum.hip", "gather.hip", "tree.hip", "pipeline.hip", "util.hip"]
 
 # -ffp-contract=off: the sums are adds only, but nothing may ever be fused.
 # -packed-fp32-ops off: keep the compiler from forming v_pk_add_f32 out of the
@@ -62,6 +62,22 @@ def build(verbose: bool = False, jobs: int = 4) -> str:
     return LIB_PATH
 
 
+def build_probe(verbose: bool = False) -> str:
+    """Compile the benchmark's measuring kernels (benchlib/probe.hip) into their own library,
+    benchlib/libtccl_probe.so: they are loaded by bench.py only and are no part of the product."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "benchlib", "probe.hip")
+    out = os.path.join(root, "benchlib", "libtccl_probe.so")
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", src, "-o", out + ".tmp"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on probe.hip:\n{proc.stdout}\n{proc.stderr}")
+    os.replace(out + ".tmp", out)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 def build_c_client(verbose: bool = False) -> str:
     """Compile the plain C client of the library (tests/c_client) next to its source."""
     root = os.path.dirname(HERE)
@@ -82,5 +98,6 @@ def build_c_client(verbose: bool = False) -> str:
 
 if __name__ == "__main__":
     build(verbose=True)
+    build_probe(verbose=True)
     build_c_client(verbose=True)
     sys.exit(0)

@@ -36,8 +36,8 @@ struct Shape {
 //   nvec      -- 16-byte vectors of output the launch produces (per row for the gather)
 //   nsrc      -- source streams read per output vector
 //   rows      -- rows of nvec vectors each that share the grid (gather), else 1
-//   is_copy   -- a pure copy: large ones get their own defaults (one workgroup per compute
-//                unit, streaming loads and stores), worth 15-20 % on this memory system
+//   is_copy   -- a pure copy: from 8 MiB they get their own defaults (one or two workgroups per
+//                compute unit, four vectors per lane, streaming loads and stores)
 Shape resolve_shape(const tccl_launch_cfg *cfg, size_t nvec, int nsrc, int rows, bool is_copy = false);
 
 } // namespace tccl

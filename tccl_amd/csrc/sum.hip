@@ -240,9 +240,13 @@ extern "C" int tccl_reduce_scatter_sum_ex(const void *const *bufs, int world, in
     const int esize = dtype_size(dtype);
     if (esize == 0 || bufs == nullptr || world < 1 || world > TCCL_MAX_WORLD || rank < 0 || rank >= world)
         return TCCL_EINVAL;
+    // Every rank's share must be the same whole number of 16-byte vectors (the reference asserts
+    // numel % (8 * world) == 0, triton_reduce_scatter.py:101-104): the answer is the same for
+    // every rank, and no element is left out.
+    if (numel_total % static_cast<size_t>(world) != 0) return TCCL_EALIGN;
     const size_t per_rank = numel_total / static_cast<size_t>(world);
+    if ((per_rank * static_cast<size_t>(esize)) % kVecBytes != 0) return TCCL_EALIGN;
     const size_t byte_off = static_cast<size_t>(rank) * per_rank * static_cast<size_t>(esize);
-    if (byte_off % kVecBytes != 0) return TCCL_EALIGN;
     const void *shifted[TCCL_MAX_WORLD];
     for (int i = 0; i < world; ++i) {
         if (bufs[i] == nullptr) return TCCL_EINVAL;

@@ -9,7 +9,11 @@ rank, as the reference counts them) plus the algorithmic HBM GB/s, after a warm-
 with HIP events on the launch stream.
 
     python -m tccl_amd.harness all_reduce|reduce_scatter|all_gather|double_tree|double_tree_pipelined|
-                               two_shot|two_shot_world [--world 8] [--max-elems N]
+                               two_shot|two_shot_world [--world 8] [--max-elems N] [--compare] [--plot out.png]
+
+``--plot`` draws what the reference's notebook draws (plot.ipynb: message size against rate, both
+axes logarithmic, one curve per implementation) from the lines just printed, with the axis in
+GB/s as measured (the notebook multiplies its GB/s by 1e6 and calls them B/s).
 """
 from __future__ import annotations
 
@@ -17,7 +21,46 @@ import argparse
 import ctypes
 import sys
 
+import re
+from typing import List, Optional, Tuple
+
 REPS = 10          # as in the reference
+
+_LINE = re.compile(r"^(?P<name>\S+) (?P<bytes>\d+) (?P<rate>[0-9.]+(?:e[+-]?\d+)?|inf|nan) GB/s")
+
+
+def parse_line(line: str) -> Optional[Tuple[str, int, float]]:
+    """``"<name> <bytes> <rate> GB/s ..."`` -> (name, bytes, rate); None for any other line."""
+    m = _LINE.match(line.strip())
+    if not m:
+        return None
+    return m.group("name"), int(m.group("bytes")), float(m.group("rate"))
+
+
+def plot(lines: List[str], path: str, title: str) -> None:
+    """Message size against rate, both axes logarithmic, one curve per name."""
+    import matplotlib
+    matplotlib.use("Agg")
+    import matplotlib.pyplot as plt
+    curves = {}
+    for ln in lines:
+        rec = parse_line(ln)
+        if rec is not None:
+            curves.setdefault(rec[0], []).append(rec[1:])
+    fig, ax = plt.subplots(figsize=(7, 4.5))
+    for name, pts in curves.items():
+        pts.sort()
+        ax.plot([p[0] for p in pts], [p[1] for p in pts], marker="o", markersize=3, label=name)
+    ax.set_xscale("log", base=2)
+    ax.set_yscale("log")
+    ax.set_xlabel("input bytes per rank")
+    ax.set_ylabel("GB/s of input bytes per rank")
+    ax.set_title(title)
+    ax.grid(True, which="both", linewidth=0.3)
+    ax.legend()
+    fig.tight_layout()
+    fig.savefig(path, dpi=120)
+    plt.close(fig)
 
 
 def main(argv=None) -> int:
@@ -27,6 +70,7 @@ def main(argv=None) -> int:
     p.add_argument("--world", type=int, default=8)
     p.add_argument("--max-elems", type=int, default=256 * 1024 * 1024 // 2,
                    help="largest element count per rank (bf16); halved down to 2,048")
+    p.add_argument("--plot", metavar="PNG", help="also draw the curves (log-log, GB/s) into this file")
     p.add_argument("--compare", action="store_true",
                    help="also time the same operation written with torch's own GPU kernels, as the second "
                         "line per size (the place the reference gives to NCCL)")
@@ -77,6 +121,12 @@ def main(argv=None) -> int:
             acc += b
         return acc.to(view.dtype)
 
+    printed: List[str] = []
+
+    def emit(line: str) -> None:
+        printed.append(line)
+        print(line, flush=True)
+
     size = args.max_elems
     while size >= 2048:
         size = size // (8 * world) * (8 * world)     # whole 16-byte vectors per rank share, whatever --max-elems was
@@ -100,7 +150,7 @@ def main(argv=None) -> int:
             line += f"  (HBM {algo_bytes(size) / per_call_ms / 1e6:.1f} GB/s, {per_call_ms * 1e3:.1f} us)"
         else:
             line += f"  ({per_call_ms * 1e3:.1f} us)"
-        print(line, flush=True)
+        emit(line)
         if args.compare:
             torch_eager(view)
             lib.tccl_event_record(start, stream)
@@ -110,12 +160,15 @@ def main(argv=None) -> int:
             lib.tccl_event_synchronize(stop)
             lib.tccl_event_elapsed_ms(start, stop, ctypes.byref(ms))
             t_ms = ms.value / REPS
-            print(f"torch {size * 2} {size * 2 / t_ms / 1e6:.3f} GB/s  ({t_ms * 1e3:.1f} us)", flush=True)
+            emit(f"torch {size * 2} {size * 2 / t_ms / 1e6:.3f} GB/s  ({t_ms * 1e3:.1f} us)")
         size //= 2
     if args.op in ("double_tree_pipelined", "two_shot_world"):
         expired = tccl_amd.signal_pad_timeouts(group)
         print(f"expired waits: {expired}", flush=True)
     tccl_amd.unregister(group)
+    if args.plot:
+        plot(printed, args.plot, f"{args.op}, {world} virtual ranks on one MI355X")
+        print(f"plot written to {args.plot}", flush=True)
     return 0
 
 

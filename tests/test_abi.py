@@ -57,7 +57,10 @@ def test_argument_checks_return_codes_without_launching():
     assert lib.tccl_all_reduce_sum(good, 2, out, 0, 0, None) == 0            # empty input: nothing to do
     assert lib.tccl_reduce_scatter_sum(good, 2, 2, out, 64, 0, None) == -1   # rank out of range
     assert lib.tccl_reduce_scatter_sum(good, 2, -1, out, 64, 0, None) == -1
-    assert lib.tccl_reduce_scatter_sum(good, 2, 1, out, 8, 0, None) == -2    # share not 16-byte aligned
+    assert lib.tccl_reduce_scatter_sum(good, 2, 1, out, 8, 0, None) == -2    # share not 16-byte aligned ...
+    assert lib.tccl_reduce_scatter_sum(good, 2, 0, out, 8, 0, None) == -2    # ... for every rank alike
+    assert lib.tccl_reduce_scatter_sum(good, 2, 0, out, 17, 0, None) == -2   # not a multiple of world
+    assert lib.tccl_reduce_scatter_sum(good, 2, 1, out, 4, 1, None) == -2    # fp32: a share of 2 elements is 8 bytes
     assert lib.tccl_reduce_scatter_sum(good, 2, 1, out, 0, 0, None) == 0
     assert lib.tccl_all_gather(good, 2, out, 24, None) == -2
     assert lib.tccl_all_gather(good, 0, out, 32, None) == -1
@@ -118,19 +121,34 @@ def test_argument_checks_return_codes_without_launching():
     assert static(good, None, 2, 64, 0, ctypes.byref(_lib.PipelineCfg(2 * 1024 + 1, 0, 0, 0)), None) == _lib.TCCL_ESCRATCH
     assert static(good, None, 2, 0, 0, None, None) == 0
     assert lib.tccl_timeout_flag_create(None) == -1 and lib.tccl_timeout_flag_destroy(None) == -1
-    assert lib.tccl_probe_read(good, 2, 64, None, None) == -1
-    assert lib.tccl_probe_read(good, 9, 64, out, None) == -1
-    assert lib.tccl_probe_read(null, 2, 64, out, None) == -1
-    assert lib.tccl_probe_read(odd, 2, 64, out, None) == -2
-    assert lib.tccl_probe_read(good, 2, 24, out, None) == -2
-    assert lib.tccl_probe_read(good, 2, 0, out, None) == 0
-    assert lib.tccl_probe_write(None, 64, None) == -1
-    assert lib.tccl_probe_write(out, 24, None) == -2
-    assert lib.tccl_probe_write(out, 0, None) == 0
     n = ctypes.c_uint(0)
     assert lib.tccl_signal_pad_timeouts(None, 4096, ctypes.byref(n), None) == -1
     assert lib.tccl_signal_pad_timeouts(ctypes.c_void_p(0x5000), 8, ctypes.byref(n), None) == -1
     assert lib.tccl_signal_pad_timeouts(ctypes.c_void_p(0x5000), 4096, None, None) == -1
+
+
+def test_probe_library_is_separate_and_checks_its_arguments():
+    """The benchmark's measuring kernels live in their own library; the product exports none of them."""
+    from benchlib import probe
+    plib = probe.load()
+    lib = tccl_amd.load_library()
+    for name in probe.SIGNATURES:
+        assert not hasattr(lib, name), f"{name} is exported by the product library"
+    good = _lib.ptr_array([0x1000, 0x2000])
+    odd = _lib.ptr_array([0x1000, 0x2008])
+    null = _lib.ptr_array([0x1000, None])
+    out = ctypes.c_void_p(0x3000)
+    assert plib.tccl_probe_read(good, 2, 64, None, None) == -1
+    assert plib.tccl_probe_read(good, 9, 64, out, None) == -1
+    assert plib.tccl_probe_read(null, 2, 64, out, None) == -1
+    assert plib.tccl_probe_read(odd, 2, 64, out, None) == -2
+    assert plib.tccl_probe_read(good, 2, 24, out, None) == -2
+    assert plib.tccl_probe_read(good, 2, 0, out, None) == 0
+    assert plib.tccl_probe_write(None, 64, None) == -1
+    assert plib.tccl_probe_write(out, 24, None) == -2
+    assert plib.tccl_probe_write(out, 0, None) == 0
+    assert plib.tccl_probe_placement(None, 8, 0, None) == -1
+    assert plib.tccl_probe_placement(out, 0, 0, None) == -1
 
 
 def test_missing_library_fails_loudly(monkeypatch):

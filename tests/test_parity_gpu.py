@@ -236,16 +236,19 @@ def test_all_reduce_sweep_sizes(world, _gpu_hygiene, c_oracle):
         nbytes *= 4
 
 
-def test_all_reduce_256mib_per_buffer(_gpu_hygiene, c_oracle):
-    """Largest sweep point: 8 x 256 MiB (offsets beyond 2^31 bytes in total)."""
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_all_reduce_256mib_per_buffer(world, _gpu_hygiene, c_oracle):
+    """Largest sweep point for every world of the sweep: W x 256 MiB against the oracle (offsets
+    beyond 2^31 bytes in total at W=8; at W=2 the launch plan is the one for few sources: a single
+    launch over 16 KiB tiles; at W=4 and 8, four and four slices of full-size tiles)."""
     n = (256 << 20) // 2
     torch.manual_seed(0)
     base = torch.randn(n, dtype=torch.bfloat16)
-    bufs = [base.roll(r * 1_000_003) for r in range(8)]
+    bufs = [base.roll(r * 1_000_003) for r in range(world)]
     g = upload(_gpu_hygiene, bufs)
-    out = tccl_amd.one_shot_all_reduce(g.tensor(0))
+    out = tccl_amd.one_shot_all_reduce(g.tensor(world - 1))
     want = oracle_sum(c_oracle, bufs)
-    assert_bit_equal(out, want, "256 MiB")
+    assert_bit_equal(out, want, f"W={world} x 256 MiB")
 
 
 def test_launches_follow_the_current_stream(_gpu_hygiene, c_oracle):
@@ -782,8 +785,10 @@ def test_plain_c_client():
 
 def test_probe_kernels_touch_what_they_say(_gpu_hygiene):
     """The measuring kernels: the read probe stores nothing (sources and sink unchanged, for
-    every world and for ragged sizes), the write probe fills exactly the bytes it is given."""
-    lib = tccl_amd.load_library()
+    every world and for ragged sizes), the write probe fills exactly the bytes it is given, the
+    placement probe reports one record per workgroup."""
+    from benchlib import probe
+    lib = probe.load()
     for world, nbytes in [(1, 16), (3, 128 * 1024 + 48), (8, 5 * 128 * 1024 * 512 // 4 + 16), (8, 64 << 20)]:
         numel = nbytes // 2
         bufs = [torch.randn(numel, dtype=torch.float32, device=DEV).to(torch.bfloat16) for _ in range(world)]
@@ -803,3 +808,9 @@ def test_probe_kernels_touch_what_they_say(_gpu_hygiene):
         assert bool((region[:guard] == 0xAB).all()) and bool((region[guard + nbytes:] == 0xAB).all())
         words = region[guard:guard + nbytes].view(torch.int32)
         assert bool((words[0::4] == 0x3F803F80).all()) and bool((words[3::4] == 0x3F803F80).all())
+    assert lib.tccl_probe_empty(stream()) == 0
+    where = torch.full((2 * 512,), -1, dtype=torch.int32, device=DEV)
+    assert lib.tccl_probe_placement(where.data_ptr(), 512, 100, stream()) == 0
+    torch.cuda.synchronize()
+    xcd = where[1::2] & 15
+    assert bool((where != -1).all()) and int(xcd.max()) <= 7
