@@ -46,7 +46,7 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "headline_traffic.json")
 ONLY_OPS = ["all_reduce", "all_reduce_rotated", "probe_read", "probe_write", "reduce_scatter_bf16", "reduce_scatter_f32",
             "all_gather_bf16", "all_gather_f32", "all_gather_int8", "tree_reduce_c0", "tree_reduce_c1",
             "tree_reduce_c2", "tree_copy_1", "tree_copy_2", "double_tree_level", "double_tree_pipelined",
-            "double_tree_pipelined_drawn", "two_shot", "two_shot_drawn", "copy_calibration", "placement", "ceilings"]
+            "double_tree_pipelined_drawn", "two_shot", "two_shot_drawn", "copy_calibration", "placement", "ceilings", "phase_timing"]
 
 
 def parse_args():
@@ -400,6 +400,8 @@ def cold_ceilings(torch, lib, plib, device):
     W = 64 << 20
     _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_write(base + k * W, W, s), 64), 128, 64)
     out["write_64MiB_128KiB_tiles_gbs"] = round(W / (ms * 1e-3) / 1e9, 1)
+    _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_write_small(base + k * W, W, s), 64), 128, 64)
+    out["write_64MiB_32KiB_tiles_gbs"] = round(W / (ms * 1e-3) / 1e9, 1)
     C = 128 << 20
     _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_copy(base + (2 * k) * C, base + (2 * k + 1) * C, C, s), 16), 32, 16)
     out["copy_128MiB_gbs"] = round(2 * C / (ms * 1e-3) / 1e9, 1)
@@ -409,9 +411,41 @@ def cold_ceilings(torch, lib, plib, device):
     return out
 
 
+def phase_timing(torch, tccl_amd, plib, device, launches=48):
+    """When do the workgroups of the large all-reduce finish reading and writing?  The kernel's
+    shape with wall-clock stamps per workgroup, rotated over 8 buffer sets; printed per XCD and
+    for the first and the second workgroup that a compute unit receives (workgroups b and b + 256)."""
+    noise = Noise(torch, device)
+    numel = BYTES_PER_BUF // 2
+    gs = [make_world(tccl_amd, torch, noise, WORLD, numel, torch.bfloat16, device, salt=9 * k) for k in range(8)]
+    outs = [torch.empty(numel, dtype=torch.bfloat16, device=device) for _ in range(8)]
+    ntiles = BYTES_PER_BUF // (128 << 10)
+    stamps = torch.zeros((launches, ntiles, 3), dtype=torch.int64, device=device)
+    s = raw_stream(torch)
+    for i in range(launches):
+        assert plib.tccl_probe_sum_timed(gs[i % 8].ptr_array, outs[i % 8].data_ptr(), BYTES_PER_BUF, stamps[i].data_ptr(), s) == 0
+    torch.cuda.synchronize()
+    t = stamps[16:].cpu().double()                            # skip the first 16 launches
+    t = (t - t[:, :, 0].min(dim=1, keepdim=True)[0].unsqueeze(-1)) * 0.01       # us after the launch's first start
+    b = torch.arange(ntiles)
+    print(f"W=8 x 64 MiB bf16, {ntiles} tiles of 128 KiB, mean over {t.shape[0]} launches rotated over 8 buffer sets; "
+          f"span {float(t[:, :, 2].max(dim=1)[0].mean()):.2f} us; times in us after the launch's first workgroup started")
+    print("XCD  workgroup on its unit   read-end mean   read-end max   write-end mean   write-end max")
+    for x in range(8):
+        for second in (0, 1):
+            sel = (b % 8 == x) & ((b >= ntiles // 2) == bool(second))
+            rd, wr = t[:, sel, 1], t[:, sel, 2]
+            print(f"{x:3d}  {'second' if second else 'first ':6s}              {float(rd.mean()):10.2f}   {float(rd.max(dim=1)[0].mean()):12.2f}   "
+                  f"{float(wr.mean()):13.2f}   {float(wr.max(dim=1)[0].mean()):12.2f}")
+    for g in gs:
+        tccl_amd.unregister(g)
+
+
 def run_only(args, torch, tccl_amd, lib, plib, device):
     if args.only == "placement":
         return placement(torch, plib, device)
+    if args.only == "phase_timing":
+        return phase_timing(torch, tccl_amd, plib, device)
     if args.only == "ceilings":
         print(json.dumps({"only": "ceilings", **cold_ceilings(torch, lib, plib, device)}), flush=True)
         return
@@ -505,10 +539,22 @@ def sweep(torch, tccl_amd, lib, noise, device):
 
 # ------------------------------------------------------------------------------------------ other ops
 
-def other_ops(torch, tccl_amd, lib, plib, noise, device):
+MIB = 1 << 20
+# bytes read and written per launch (algorithmic), for the memory-system bound of each operation
+READS_WRITES = {
+    "reduce_scatter_bf16": (128 * MIB, 16 * MIB), "reduce_scatter_f32": (256 * MIB, 32 * MIB),
+    "all_gather_bf16": (128 * MIB, 128 * MIB), "all_gather_f32": (256 * MIB, 256 * MIB), "all_gather_int8": (64 * MIB, 64 * MIB),
+    "tree_reduce_c0": (128 * MIB, 128 * MIB), "tree_reduce_c1": (256 * MIB, 128 * MIB), "tree_reduce_c2": (384 * MIB, 128 * MIB),
+    "tree_copy_1": (128 * MIB, 128 * MIB), "tree_copy_2": (128 * MIB, 256 * MIB),
+}
+
+
+def other_ops(torch, tccl_amd, lib, plib, noise, device, ceilings=None):
     """The other operations of the path at their full benchmark shapes: GB/s on algorithmic bytes
     from HIP events (30 launches after 6 warm-ups), every one rotated over enough disjoint buffers
-    that nothing is served from the 256 MB memory-side cache."""
+    that nothing is served from the 256 MB memory-side cache.  `of_bound`: the time a pure read pass
+    plus a pure write pass of the same bytes would take at the cold rates measured in this run
+    (cold_memory_ceilings: multi-stream read, write), divided by the operation's own time."""
     out = {}
     ops = Ops(torch, tccl_amd, lib, plib, noise, device)
     for name in ("reduce_scatter_bf16", "reduce_scatter_f32", "all_gather_bf16", "all_gather_f32", "all_gather_int8",
@@ -517,6 +563,10 @@ def other_ops(torch, tccl_amd, lib, plib, noise, device):
         _, ms = time_steps(torch, lib, fn, 30, 6)
         out[name] = {"gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "us": round(ms * 1e3, 2),
                      "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 3)}
+        if ceilings and "read_8_streams_128KiB_tiles_gbs" in ceilings:
+            rd, wr = READS_WRITES[name]
+            bound_us = rd / ceilings["read_8_streams_128KiB_tiles_gbs"] / 1e3 + wr / ceilings["write_64MiB_32KiB_tiles_gbs"] / 1e3
+            out[name]["of_bound"] = round(bound_us / (ms * 1e3), 3)
         ops.close()
     # whole double-tree all-reduce, W=8 x 256 MiB: level schedule, pipelined single launch (both chunk sizes, both bindings)
     for how, key in (("level", "double_tree_w8_256MiB_level_schedule_ms"),
@@ -765,7 +815,7 @@ def main():
 
     if not args.no_other_ops:
         try:
-            result["other_ops"] = other_ops(torch, tccl_amd, lib, plib, noise, device)
+            result["other_ops"] = other_ops(torch, tccl_amd, lib, plib, noise, device, result.get("cold_memory_ceilings"))
         except RuntimeError as e:        # the headline must still be printed
             result["other_ops"] = {"error": str(e)[:200]}
 

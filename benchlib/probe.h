@@ -19,12 +19,18 @@ extern "C" {
 int tccl_probe_read(const void *const *bufs, int world, size_t bytes_per_buffer, void *sink, void *stream);
 /* The write half: fills `bytes` at dst with a pattern, 32 stores per lane back to back. */
 int tccl_probe_write(void *dst, size_t bytes, void *stream);
+/* The same fill in 32 KiB tiles: the fastest way found to write HBM. */
+int tccl_probe_write_small(void *dst, size_t bytes, void *stream);
 /* One contiguous range read front to back by the whole GPU (grid-stride, streaming loads): the
  * fastest way found to read HBM, the reference point for every read rate in the benchmark. */
 int tccl_probe_read_dense(const void *buf, size_t bytes, void *sink, void *stream);
 /* A plain copy in the launch shape that is fastest on uncached data: the reference point for the
  * copies (all-gather, tree copy step). */
 int tccl_probe_copy(const void *src, void *dst, size_t bytes, void *stream);
+/* The large all-reduce's kernel shape (8 bf16 sources, one 128 KiB tile per workgroup) with time
+ * stamps: stamps[3*b + 0..2] = 100 MHz wall clock of workgroup b at its start, at the end of its
+ * read phase and at the end of its writes. */
+int tccl_probe_sum_timed(const void *const *bufs, void *out, size_t bytes_per_buffer, long long *stamps, void *stream);
 /* One empty kernel: what a timed single launch costs when the kernel does nothing. */
 int tccl_probe_empty(void *stream);
 /* out[2*b] = HW_REG_HW_ID, out[2*b+1] = HW_REG_XCC_ID of workgroup b of a grid of `workgroups`

@@ -13,8 +13,10 @@ _PP = ctypes.POINTER(ctypes.c_void_p)
 SIGNATURES = {
     "tccl_probe_read": (_I, [_PP, _I, _SZ, _P, _P]),
     "tccl_probe_write": (_I, [_P, _SZ, _P]),
+    "tccl_probe_write_small": (_I, [_P, _SZ, _P]),
     "tccl_probe_read_dense": (_I, [_P, _SZ, _P, _P]),
     "tccl_probe_copy": (_I, [_P, _P, _SZ, _P]),
+    "tccl_probe_sum_timed": (_I, [_PP, _P, _SZ, _P, _P]),
     "tccl_probe_empty": (_I, [_P]),
     "tccl_probe_placement": (_I, [_P, _I, _I, _P]),
 }
