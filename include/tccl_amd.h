@@ -304,6 +304,34 @@ int tccl_two_shot_all_reduce_static(void *const *bufs, void *const *outs, int wo
 int tccl_timeout_flag_create(uint32_t **flag_out);
 int tccl_timeout_flag_destroy(uint32_t *flag);
 
+/* Buffers that several processes on one GPU can map: what the reference gets from
+ * _SymmetricMemory.empty_strided_p2p (triton_one_shot_all_reduce_no_128.py:116-122) and
+ * rendezvous (:82).  tccl_symm_alloc returns a zero-filled device allocation of its own (below
+ * 2 GiB); tccl_ipc_export writes its 64-byte handle, which the host side carries to the peers;
+ * tccl_ipc_open maps a peer's allocation into this process and returns its address here, good for
+ * every pointer table of this header; tccl_ipc_close unmaps it.  These four calls allocate, map or
+ * synchronise: they belong to set-up, not to the hot path. */
+#define TCCL_IPC_HANDLE_BYTES 64
+int tccl_symm_alloc(size_t bytes, void **ptr_out);
+int tccl_symm_free(void *ptr);
+int tccl_ipc_export(void *ptr, unsigned char *handle_out /* TCCL_IPC_HANDLE_BYTES */);
+int tccl_ipc_open(const unsigned char *handle /* TCCL_IPC_HANDLE_BYTES */, void **ptr_out);
+int tccl_ipc_close(void *ptr);
+
+/* The reference's blockwise_barrier (triton_barrier.py:39-142) as a launch of its own, one per
+ * rank: rank `rank`'s kernel raises slot `block * world + rank` in every peer's pad and waits for
+ * slot `block * world + peer` of its own pad, which it lowers again; `blocks` independent rows of
+ * slots (the reference has one per workgroup of the collective's kernel).  Everything this rank
+ * enqueued on `stream` before the call is complete and visible to the peers' work that follows
+ * their call, and the other way round (the guarantee of triton_barrier.py:56-66); called again
+ * after a collective it is the trailing barrier the reference lacks.  signal_pads: HOST array of
+ * `world` device pointers, own pad at index `rank`, the peers' pads as opened with tccl_ipc_open;
+ * each zero-filled before the first use, pad_bytes >= 4 * blocks * world, left zero-filled by every
+ * completed barrier.  Waits are bounded: after spin_limit polls (0 = about a second) a lane sets
+ * *timeout_flag (if given; pinned host memory, tccl_timeout_flag_create) and gives up. */
+int tccl_blockwise_barrier(void *const *signal_pads, size_t pad_bytes, int world, int rank, int blocks,
+                           unsigned spin_limit, uint32_t *timeout_flag, void *stream);
+
 /* HIP-event helpers so a host language without HIP bindings can time launches on the very
  * stream they run on.  No counterpart in the reference (it times with torch.cuda.Event,
  * triton_reduce_scatter.py:216-226). */

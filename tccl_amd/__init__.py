@@ -7,7 +7,7 @@ from .collectives import (DoubleTreePlan, all_gather, all_reduce, double_tree_al
                           one_shot_all_reduce, one_shot_reduce_scatter, reduce_scatter, signal_pad_timeouts, two_shot_all_reduce,
                           two_shot_all_reduce_world)
 from .symm import SymmGroup, SymmHandle, empty_world, register, rendezvous, unregister
-from . import spmd, tree
+from . import ipc, spmd, tree
 from .tree import build_double_tree, build_tree, get_parents_and_children
 
 __all__ = [
@@ -15,5 +15,5 @@ __all__ = [
     "one_shot_all_reduce", "one_shot_reduce_scatter", "one_shot_all_gather", "double_tree_all_reduce",
     "double_tree_all_reduce_world", "signal_pad_timeouts", "two_shot_all_reduce_world", "DoubleTreePlan", "reduce_scatter", "all_gather", "two_shot_all_reduce", "all_reduce",
     "SymmGroup", "SymmHandle", "empty_world", "register", "rendezvous", "unregister",
-    "spmd", "tree", "build_tree", "build_double_tree", "get_parents_and_children",
+    "ipc", "spmd", "tree", "build_tree", "build_double_tree", "get_parents_and_children",
 ]

@@ -16,6 +16,7 @@ ABI_VERSION = 2
 TCCL_OK, TCCL_EINVAL, TCCL_EALIGN, TCCL_EPOW2, TCCL_ESCRATCH, TCCL_ETIMEOUT = 0, -1, -2, -3, -4, -5
 MAX_WORLD = 8
 MAX_JOBS = 8
+IPC_HANDLE_BYTES = 64
 
 TCCL_BF16 = 0
 TCCL_F32 = 1
@@ -89,6 +90,12 @@ SIGNATURES = {
     "tccl_two_shot_all_reduce_static": (_I, [_PP, _PP, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
     "tccl_timeout_flag_create": (_I, [ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32))]),
     "tccl_timeout_flag_destroy": (_I, [ctypes.POINTER(ctypes.c_uint32)]),
+    "tccl_symm_alloc": (_I, [_SZ, _PP]),
+    "tccl_symm_free": (_I, [_P]),
+    "tccl_ipc_export": (_I, [_P, ctypes.POINTER(ctypes.c_ubyte)]),
+    "tccl_ipc_open": (_I, [ctypes.POINTER(ctypes.c_ubyte), _PP]),
+    "tccl_ipc_close": (_I, [_P]),
+    "tccl_blockwise_barrier": (_I, [_PP, _SZ, _I, _I, _I, ctypes.c_uint, ctypes.POINTER(ctypes.c_uint32), _P]),
     "tccl_double_tree_plan_create": (_I, [_PP, _PP, _I, _SZ, _I, _SZ, _PP]),
     "tccl_plan_launch": (_I, [_P, _P]),
     "tccl_plan_destroy": (_I, [_P]),

@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "_obj")
 LIB_PATH = os.path.join(HERE, "libtccl_amd.so")
 
-SOURCES = ["sum.hip", "gather.hip", "tree.hip", "pipeline.hip", "util.hip"]
+SOURCES = ["sum.hip", "gather.hip", "tree.hip", "pipeline.hip", "ipc.hip", "util.hip"]
 
 # -ffp-contract=off: the sums are adds only, but nothing may ever be fused.
 # -packed-fp32-ops off: keep the compiler from forming v_pk_add_f32 out of the

@@ -1,0 +1,168 @@
+"""Symmetric buffers owned by separate processes on one GPU.
+
+The reference's ranks are processes: each allocates its buffer with
+``_SymmetricMemory.empty_strided_p2p`` (triton_one_shot_all_reduce_no_128.py:116-122) and gets
+the table of all ranks' buffer addresses from ``rendezvous`` (:82).  This module does the same
+for W processes that share one MI355X: a rank's buffer is a device allocation of its own
+(``tccl_symm_alloc``), exported as a 64-byte handle, carried to the peers through a directory
+they all see, and mapped there (``tccl_ipc_open``).  The resulting ``SymmHandle`` goes through
+the same wrappers as a group of virtual ranks (``one_shot_all_reduce``, ``reduce_scatter``,
+``all_gather``); ordering between the ranks' launches is the reference's device-side
+``blockwise_barrier`` (triton_barrier.py:39-142), one kernel launch per rank
+(``IpcWorld.barrier``), before a collective and -- what the reference lacks -- after it.
+
+    world = IpcWorld(rank, world_size, directory)          # one per process
+    tensor = world.empty(numel, torch.bfloat16)            # this rank's buffer, peers mapped
+    tensor.copy_(...)
+    world.barrier()                                        # every rank's buffer is filled
+    out = tccl_amd.one_shot_all_reduce(tensor)
+    world.barrier()                                        # every rank has read it
+    world.close()
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import time
+from typing import List, Optional
+
+import torch
+
+from . import _lib, symm
+
+_DTYPE_TYPESTR = {torch.bfloat16: None, torch.float32: "<f4", torch.int8: "|i1", torch.uint8: "|u1", torch.int16: "<i2",
+                  torch.int32: "<i4"}
+
+
+class _DeviceBlock:
+    """A raw device allocation seen through ``__cuda_array_interface__`` so that torch can wrap it."""
+
+    def __init__(self, ptr: int, nbytes: int):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 2}
+
+
+def _as_tensor(ptr: int, nbytes: int, device) -> torch.Tensor:
+    return torch.as_tensor(_DeviceBlock(ptr, nbytes), device=device)
+
+
+class IpcWorld:
+    """This process's view of W processes sharing one GPU.  ``directory`` is where the ranks leave
+    their handles for each other (any place all of them can read and write)."""
+
+    BARRIER_BLOCKS = 4
+    PAD_BYTES = 4096
+
+    def __init__(self, rank: int, world_size: int, directory: str, device="cuda:0", timeout_s: float = 60.0):
+        if not (1 <= world_size <= _lib.MAX_WORLD and 0 <= rank < world_size):
+            raise ValueError("rank/world_size out of range")
+        self.rank, self.world_size, self.directory, self.timeout_s = rank, world_size, directory, timeout_s
+        self.device = torch.device(device)
+        self.lib = _lib.load()
+        self._allocs: List[int] = []          # own allocations
+        self._opened: List[int] = []          # peers' allocations mapped here
+        self._count = 0
+        self._host_barriers = 0
+        self._flag = ctypes.POINTER(ctypes.c_uint32)()
+        _lib.check("tccl_timeout_flag_create", self.lib.tccl_timeout_flag_create(ctypes.byref(self._flag)))
+        # signal pads: one per rank, every rank maps all of them
+        self._pad_ptrs = self._exchange(self._alloc(self.PAD_BYTES), "pad")
+        self._pad_array = _lib.ptr_array(self._pad_ptrs)
+
+    # ---- plumbing
+    def _alloc(self, nbytes: int) -> int:
+        p = ctypes.c_void_p()
+        _lib.check("tccl_symm_alloc", self.lib.tccl_symm_alloc(nbytes, ctypes.byref(p)))
+        self._allocs.append(p.value)
+        return p.value
+
+    def _wait_for(self, path: str) -> bytes:
+        t_end = time.monotonic() + self.timeout_s
+        while time.monotonic() < t_end:
+            try:
+                with open(path, "rb") as f:
+                    data = f.read()
+                if data:
+                    return data
+            except OSError:
+                pass
+            time.sleep(0.002)
+        raise TimeoutError(f"rank {self.rank}: {path} did not appear within {self.timeout_s} s")
+
+    def _publish(self, name: str, data: bytes) -> None:
+        tmp = os.path.join(self.directory, f".{name}.tmp{self.rank}")
+        with open(tmp, "wb") as f:
+            f.write(data)
+        os.replace(tmp, os.path.join(self.directory, name))          # appears whole or not at all
+
+    def _exchange(self, own_ptr: int, what: str) -> List[int]:
+        """Export own_ptr, collect everybody's handle, map the peers'; addresses in rank order."""
+        tag = f"{what}{self._count}"
+        self._count += 1
+        handle = (ctypes.c_ubyte * _lib.IPC_HANDLE_BYTES)()
+        _lib.check("tccl_ipc_export", self.lib.tccl_ipc_export(own_ptr, handle))
+        self._publish(f"{tag}.rank{self.rank}", bytes(handle))
+        ptrs = []
+        for r in range(self.world_size):
+            if r == self.rank:
+                ptrs.append(own_ptr)
+                continue
+            raw = self._wait_for(os.path.join(self.directory, f"{tag}.rank{r}"))
+            h = (ctypes.c_ubyte * _lib.IPC_HANDLE_BYTES).from_buffer_copy(raw)
+            p = ctypes.c_void_p()
+            _lib.check("tccl_ipc_open", self.lib.tccl_ipc_open(h, ctypes.byref(p)))
+            self._opened.append(p.value)
+            ptrs.append(p.value)
+        return ptrs
+
+    # ---- what a per-rank program uses
+    def empty(self, numel: int, dtype: torch.dtype) -> torch.Tensor:
+        """This rank's buffer of a symmetric allocation (zero-filled), registered with the peers'
+        mapped buffers as one group: collective, every rank must make the same calls in the same
+        order (as with ``empty_strided_p2p`` followed by ``rendezvous``)."""
+        esize = torch.empty(0, dtype=dtype).element_size()
+        nbytes = numel * esize
+        own = self._alloc(max(nbytes, 16))
+        ptrs = self._exchange(own, "buf")
+        tensor = _as_tensor(own, nbytes, self.device).view(dtype)
+        symm.register_remote(tensor, self.rank, ptrs)
+        return tensor
+
+    def host_barrier(self) -> None:
+        """All ranks have reached this point on the host (through the directory)."""
+        tag = f"host{self._host_barriers}"
+        self._host_barriers += 1
+        self._publish(f"{tag}.rank{self.rank}", b"1")
+        for r in range(self.world_size):
+            self._wait_for(os.path.join(self.directory, f"{tag}.rank{r}"))
+
+    def barrier(self, spin_limit: int = 0) -> None:
+        """The reference's ``blockwise_barrier`` on torch's current stream: everything this rank
+        enqueued before is complete before any rank's later work starts.  Asynchronous; a wait
+        that expires is reported by ``check()``."""
+        stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        rc = self.lib.tccl_blockwise_barrier(self._pad_array, self.PAD_BYTES, self.world_size, self.rank,
+                                             self.BARRIER_BLOCKS, spin_limit, self._flag, stream)
+        _lib.check("tccl_blockwise_barrier", rc)
+
+    def check(self) -> None:
+        """Synchronise and raise if a barrier wait expired (a peer never arrived)."""
+        torch.cuda.synchronize(self.device)
+        if self._flag[0] != 0:
+            self._flag[0] = 0
+            raise _lib.TcclError("tccl_blockwise_barrier", _lib.TCCL_ETIMEOUT, "a peer did not reach the barrier in time")
+
+    def close(self) -> None:
+        """Unmap the peers' buffers and free the own ones (after a last host barrier, so that nobody
+        unmaps what a peer is still using)."""
+        torch.cuda.synchronize(self.device)
+        self.host_barrier()
+        for p in self._opened:
+            self.lib.tccl_ipc_close(p)
+        self._opened = []
+        self.host_barrier()
+        for p in self._allocs:
+            self.lib.tccl_symm_free(p)
+        self._allocs = []
+        if self._flag:
+            self.lib.tccl_timeout_flag_destroy(self._flag)
+            self._flag = ctypes.POINTER(ctypes.c_uint32)()

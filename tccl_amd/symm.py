@@ -140,6 +140,43 @@ def register(tensors: Sequence[torch.Tensor]) -> SymmGroup:
     return group
 
 
+class RemoteSymmGroup(SymmGroup):
+    """A group of which this process owns one buffer; the other ranks' buffers belong to other
+    processes and are known by the addresses they are mapped at here (``tccl_amd.ipc``).  Serves
+    the per-rank collectives (all-reduce, reduce-scatter, all-gather), which need the address
+    table, the rank and the world size only."""
+
+    def __init__(self, own: torch.Tensor, rank: int, buffer_ptrs: Sequence[int]):   # noqa: super().__init__ not called
+        if not own.is_contiguous() or int(own.data_ptr()) != int(buffer_ptrs[rank]):
+            raise ValueError("the own buffer must be the whole allocation at buffer_ptrs[rank]")
+        self.tensors = [own]
+        self.world_size = len(buffer_ptrs)
+        self.buffer_ptrs = tuple(int(p) for p in buffer_ptrs)
+        self.ptr_array = _lib.ptr_array(self.buffer_ptrs)
+        self.handles = [SymmHandle(self, r) for r in range(self.world_size)]
+        self.pending_outputs = {}
+        self.pending_versions = ()
+        self.collective_number = 0
+        self._signal_pads = []
+        self._signal_pad_array = None
+        self._timeout_flag = None
+        self.own_rank = rank
+
+    def tensor(self, rank: int) -> torch.Tensor:
+        if rank != self.own_rank:
+            raise RuntimeError("only the own rank's buffer is a tensor in this process")
+        return self.tensors[0]
+
+
+def register_remote(own: torch.Tensor, rank: int, buffer_ptrs: Sequence[int]) -> RemoteSymmGroup:
+    """Declare that ``own`` is rank ``rank``'s buffer of a symmetric allocation whose other buffers
+    live in other processes and are mapped here at ``buffer_ptrs`` (rank order)."""
+    group = RemoteSymmGroup(own, rank, buffer_ptrs)
+    _registry[int(own.data_ptr())] = (weakref.ref(group), rank)
+    own._tccl_group = group           # noqa: SLF001
+    return group
+
+
 def empty_world(world_size: int, size, dtype: torch.dtype, device="cuda") -> SymmGroup:
     """Allocate one buffer per virtual rank (each a separate ``torch.empty``) and register
     the group: the single-GPU counterpart of every rank calling ``empty_strided_p2p``."""

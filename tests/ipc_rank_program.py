@@ -1,0 +1,67 @@
+"""One rank of a reference-style per-rank program, run as its own process (started by
+test_ipc_gpu.py, W of them on one GPU): allocate a symmetric buffer, fill it with the
+reference's recipe, meet the peers in the device-side barrier, run the collectives, leave the
+results where the parent can compare them with the oracle.
+
+    python ipc_rank_program.py <rank> <world> <directory> <mode>
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+import tccl_amd                       # noqa: E402
+from tccl_amd import ipc              # noqa: E402
+
+
+def save(directory, name, rank, t):
+    t = t.detach().cpu().contiguous()
+    view = {2: torch.int16, 4: torch.int32, 1: torch.int8}[t.element_size()]
+    np.save(os.path.join(directory, f"{name}.rank{rank}.npy"), t.view(view).numpy())
+
+
+def main():
+    rank, world_size, directory, mode = int(sys.argv[1]), int(sys.argv[2]), sys.argv[3], sys.argv[4]
+    world = ipc.IpcWorld(rank, world_size, directory)
+    print(f"rank {rank}: pads exchanged", flush=True)
+    if mode == "missing_peer":
+        # rank 0 waits in the barrier, nobody else comes: its wait must expire and be reported
+        if rank == 0:
+            world.barrier(spin_limit=2000)
+            try:
+                world.check()
+            except tccl_amd.TcclError as e:
+                print(f"rank 0: reported: {e}", flush=True)
+                world.host_barrier()
+                return 42
+            return 1
+        world.host_barrier()
+        return 0
+
+    numel = 8 * world_size * 4099
+    bf = world.empty(numel, torch.bfloat16)
+    fp = world.empty(numel // 2, torch.float32)
+    for round_ in range(2):
+        torch.manual_seed(100 * round_ + rank)
+        bf.copy_(torch.randn(numel, dtype=torch.bfloat16))
+        torch.manual_seed(100 * round_ + rank)
+        fp.copy_(torch.rand(numel // 2, dtype=torch.float32) * 2 - 1)
+        world.barrier()                                  # leading barrier: every rank's buffers are filled
+        save(directory, f"all_reduce_bf16.{round_}", rank, tccl_amd.one_shot_all_reduce(bf))
+        save(directory, f"reduce_scatter_bf16.{round_}", rank, tccl_amd.reduce_scatter(bf))
+        save(directory, f"all_gather_bf16.{round_}", rank, tccl_amd.all_gather(bf, world_size))
+        save(directory, f"all_reduce_f32.{round_}", rank, tccl_amd.one_shot_all_reduce(fp))
+        save(directory, f"reduce_scatter_f32.{round_}", rank, tccl_amd.reduce_scatter(fp))
+        world.barrier()                                  # trailing barrier: every rank has read them
+        world.check()
+        print(f"rank {rank}: round {round_} done", flush=True)
+    world.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -127,6 +127,28 @@ def test_argument_checks_return_codes_without_launching():
     assert lib.tccl_signal_pad_timeouts(ctypes.c_void_p(0x5000), 4096, None, None) == -1
 
 
+def test_ipc_and_barrier_entry_points_check_their_arguments():
+    lib = tccl_amd.load_library()
+    pads = _lib.ptr_array([0x5000, 0x6000])
+    p = ctypes.c_void_p()
+    h = (ctypes.c_ubyte * _lib.IPC_HANDLE_BYTES)()
+    assert lib.tccl_symm_alloc(0, ctypes.byref(p)) == -1
+    assert lib.tccl_symm_alloc(1 << 31, ctypes.byref(p)) == -1          # mapped allocations stay below 2 GiB
+    assert lib.tccl_symm_alloc(64, None) == -1
+    assert lib.tccl_symm_free(None) == -1
+    assert lib.tccl_ipc_export(None, h) == -1 and lib.tccl_ipc_open(None, ctypes.byref(p)) == -1
+    assert lib.tccl_ipc_open(h, None) == -1 and lib.tccl_ipc_close(None) == -1
+    bar = lib.tccl_blockwise_barrier
+    assert bar(None, 4096, 2, 0, 1, 0, None, None) == -1
+    assert bar(pads, 4096, 9, 0, 1, 0, None, None) == -1
+    assert bar(pads, 4096, 2, 2, 1, 0, None, None) == -1
+    assert bar(pads, 4096, 2, 0, 0, 0, None, None) == -1
+    assert bar(pads, 4, 2, 0, 1, 0, None, None) == -1                   # pad smaller than blocks x world slots
+    assert bar(_lib.ptr_array([0x5000, None]), 4096, 2, 0, 1, 0, None, None) == -1
+    assert bar(_lib.ptr_array([0x5000, 0x6004]), 4096, 2, 0, 1, 0, None, None) == -2
+    assert bar(pads, 4096, 1, 0, 1, 0, None, None) == 0                 # a world of one has nobody to wait for
+
+
 def test_probe_library_is_separate_and_checks_its_arguments():
     """The benchmark's measuring kernels live in their own library; the product exports none of them."""
     from benchlib import probe

@@ -1,0 +1,75 @@
+"""Symmetric buffers owned by separate processes on one GPU: W child processes each allocate their
+buffer, exchange IPC handles, meet in the device-side blockwise barrier (one launch per rank, as
+the reference's kernels do: triton_barrier.py:39-142) and run the collectives on the mapped
+addresses; the parent compares what every rank got with the oracle, bit for bit."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import seeded_randn, seeded_uniform
+from oracle import torch_ref
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PROGRAM = os.path.join(ROOT, "tests", "ipc_rank_program.py")
+
+
+def run_ranks(world, directory, mode, timeout=110):
+    procs = [subprocess.Popen([sys.executable, PROGRAM, str(r), str(world), str(directory), mode],
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True) for r in range(world)]
+    outs, codes = [], []
+    try:
+        for p in procs:
+            out, _ = p.communicate(timeout=timeout)
+            outs.append(out)
+            codes.append(p.returncode)
+    finally:
+        for p in procs:                      # exactly the processes started here
+            if p.poll() is None:
+                p.kill()
+                p.wait()
+    return codes, outs
+
+
+def load(directory, name, rank, dtype):
+    a = np.load(os.path.join(directory, f"{name}.rank{rank}.npy"))
+    return torch.from_numpy(a).view(dtype)
+
+
+@pytest.mark.parametrize("world", [4, 8])
+def test_collectives_across_processes(world, tmp_path):
+    assert torch.cuda.is_available()
+    print(f"ipc: {world} processes", flush=True)
+    codes, outs = run_ranks(world, tmp_path, "collectives")
+    assert codes == [0] * world, "\n".join(outs)
+    numel = 8 * world * 4099
+    per = numel // world
+    for round_ in range(2):
+        bf = seeded_randn(world, numel, seed_base=100 * round_)
+        fp = seeded_uniform(world, numel // 2, seed_base=100 * round_)
+        want_bf, want_fp = torch_ref.all_reduce(bf), torch_ref.all_reduce(fp)
+        stacked = torch.stack(bf)
+        perf = (numel // 2) // world
+        for r in range(world):
+            assert torch.equal(load(tmp_path, f"all_reduce_bf16.{round_}", r, torch.bfloat16).view(torch.int16),
+                               want_bf.view(torch.int16)), f"round {round_} rank {r}: all-reduce bf16"
+            assert torch.equal(load(tmp_path, f"reduce_scatter_bf16.{round_}", r, torch.bfloat16).view(torch.int16),
+                               want_bf[r * per:(r + 1) * per].view(torch.int16)), f"round {round_} rank {r}: reduce-scatter bf16"
+            assert torch.equal(load(tmp_path, f"all_gather_bf16.{round_}", r, torch.bfloat16).view(torch.int16),
+                               stacked.view(torch.int16)), f"round {round_} rank {r}: all-gather"
+            assert torch.equal(load(tmp_path, f"all_reduce_f32.{round_}", r, torch.float32).view(torch.int32),
+                               want_fp.view(torch.int32)), f"round {round_} rank {r}: all-reduce f32"
+            assert torch.equal(load(tmp_path, f"reduce_scatter_f32.{round_}", r, torch.float32).view(torch.int32),
+                               want_fp[r * perf:(r + 1) * perf].view(torch.int32)), f"round {round_} rank {r}: reduce-scatter f32"
+
+
+def test_barrier_with_a_missing_peer_gives_up_and_says_so(tmp_path):
+    """Failure handling forced from the host: rank 0 enters the barrier with a small spin limit and
+    no peer ever does.  Its kernel must end by itself and the rank must be told."""
+    codes, outs = run_ranks(2, tmp_path, "missing_peer", timeout=90)
+    assert codes == [42, 0], "\n".join(outs)
+    assert "did not reach the barrier" in outs[0]
