@@ -256,7 +256,7 @@ class Ops:
         gs = self._worlds(nsets, WORLD, numel, torch.bfloat16)
         outs = [torch.empty_like(g.tensor(0)) for g in gs]
         fn = Rotation(lambda k: self.tccl_amd.one_shot_all_reduce(gs[k].tensor(0), out=outs[k]), nsets)
-        return fn, nbytes, "sum_phased_kernel<Bf16Sum, 8, 1, true>"
+        return fn, nbytes, "sum_phased_skewed_kernel<Bf16Sum, 8>"
 
     def probe_read(self):
         torch = self.torch
@@ -764,7 +764,7 @@ def main():
             "traffic": traffic,
             "traffic_source": traffic_source,
             "traffic_measured_on_these_sources": traffic_current,
-            "kernel": "tccl::sum_phased_kernel<Bf16Sum, 8, 1, true>",
+            "kernel": "tccl::sum_phased_skewed_kernel<Bf16Sum, 8>",
             "avg_launch_us": round(dev_ms * 1e3, 2),
             "algorithmic_bytes": algo_bytes,
         },

@@ -92,6 +92,35 @@ sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
 }
 
+// The same launch with unequal tiles: workgroups 2p and 2p+1 share 2 * KMAX iterations, the even
+// one taking KMAX + 1 and the odd one KMAX - 1.  Workgroup b runs on XCD b mod 8, and on MI355X
+// the odd XCDs read more slowly than the even ones when the whole GPU streams from memory (their
+// L2s wait three times as long for DRAM credits; their workgroups finish a 128 KiB tile 6 us
+// later), so the launch ends when the odd XCDs do.  One iteration in 32 moved from the odd to the
+// even XCDs measured 0.7-1 % faster on one buffer set and on rotated ones; two or more lose again.
+template <class Sum, int NSRC>
+__global__ void __launch_bounds__(kPhasedBlock)
+sum_phased_skewed_kernel(SrcTable<NSRC> src, char *out, size_t bytes, size_t tail_first, size_t numel)
+{
+    constexpr int KMAX = kPhasedVecs;                                   // one vector per lane per iteration
+    constexpr size_t span = static_cast<size_t>(kPhasedBlock) * kVecBytes;
+    const size_t pair_off = static_cast<size_t>(blockIdx.x >> 1) * (2 * KMAX * span);
+    char *const dst[1] = {out};
+    if (blockIdx.x & 1) {
+        const size_t off = pair_off + (KMAX + 1) * span;
+        const size_t left = bytes > off ? bytes - off : 0;
+        constexpr size_t tile_bytes = (KMAX - 1) * span;
+        sum_tile_phased<Sum, NSRC, 1, 1, KMAX - 1, true, Sum::kPaceLoads>(
+            src.p, dst, off, static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes), KMAX - 1);
+    } else {
+        const size_t left = bytes > pair_off ? bytes - pair_off : 0;
+        constexpr size_t tile_bytes = (KMAX + 1) * span;
+        sum_tile_phased<Sum, NSRC, 1, 1, KMAX + 1, true, Sum::kPaceLoads>(
+            src.p, dst, pair_off, static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes), KMAX + 1);
+    }
+    if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
+}
+
 template <class Sum, int NSRC, int U>
 static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t numel, const tccl_launch_cfg *cfg,
                                   hipStream_t stream)
@@ -129,6 +158,9 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
     if (wgs > (static_cast<size_t>(1) << 30)) wgs = static_cast<size_t>(1) << 30; // grid dimension limit
     const size_t tile_vec = kcount * span;
     const size_t slice_vec = wgs * tile_vec;
+    // full-size tiles of many sources, launch shape left to the library: unequal tiles for even and
+    // odd XCDs (see sum_phased_skewed_kernel)
+    const bool skewed = U == 1 && NSRC >= 5 && kcount == kmax && cfg == nullptr && wgs % 2 == 0;
     const size_t tail_first = nvec * per_vec;
 
     size_t off = 0;
@@ -142,7 +174,12 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
         // the tail's element indices are relative to this launch's base pointers
         const size_t rel_first = last ? tail_first - off * per_vec : 0;
         const size_t rel_numel = last ? numel - off * per_vec : 0;
-        if (kcount == kmax)
+        if (skewed) {
+            if constexpr (U == 1 && NSRC >= 5)
+                hipLaunchKernelGGL((sum_phased_skewed_kernel<Sum, NSRC>), dim3(static_cast<unsigned>((grid + 1) / 2 * 2)),
+                                   dim3(kPhasedBlock), 0, stream, t, out + off * kVecBytes, n * kVecBytes, rel_first,
+                                   rel_numel);
+        } else if (kcount == kmax)
             hipLaunchKernelGGL((sum_phased_kernel<Sum, NSRC, U, true>), dim3(static_cast<unsigned>(grid)),
                                dim3(kPhasedBlock), 0, stream, t, out + off * kVecBytes, n * kVecBytes,
                                static_cast<int>(kcount), rel_first, rel_numel);
