@@ -92,32 +92,40 @@ sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
 }
 
-// The same launch with unequal tiles: workgroups 2p and 2p+1 share 2 * KMAX iterations, the even
-// one taking KMAX + 1 and the odd one KMAX - 1.  Workgroup b runs on XCD b mod 8, and on MI355X
-// the odd XCDs read more slowly than the even ones when the whole GPU streams from memory (their
-// L2s wait three times as long for DRAM credits; their workgroups finish a 128 KiB tile 6 us
-// later), so the launch ends when the odd XCDs do.  One iteration in 32 moved from the odd to the
-// even XCDs measured 0.7-1 % faster on one buffer set and on rotated ones; two or more lose again.
+// The same launch with unequal, interleaved tiles: workgroups 2p and 2p+1 share a region of
+// 2 * KMAX pieces (a piece = what one iteration covers, 4 KiB), the even one taking KMAX + 1 and
+// the odd one KMAX - 1 of them.  Workgroup b runs on XCD b mod 8, and on MI355X the odd XCDs read
+// more slowly than the even ones when the whole GPU streams from memory (their L2s wait three
+// times as long for DRAM credits; their workgroups finish a 128 KiB tile 6 us later), so the
+// launch ends when the odd XCDs do.  One iteration in 32 moved from the odd to the even XCDs
+// measured 0.7-1 % faster on one buffer set and on rotated ones; two or more lose again.  The two
+// take alternate pieces of their region (the even one also the last two), so that the pair works
+// on the same 8 KiB at a time: another 0.6 % on one buffer set and 1 % on rotated ones; wider
+// groups (4, 8 or 16 workgroups interleaved, of one XCD or of neighbouring ones) lose 2-4 %.
+template <int KMAX>
+struct PieceOfEvenWorkgroup { // pieces 0, 2, ..., 2 KMAX - 4, then 2 KMAX - 2 and 2 KMAX - 1
+    static constexpr uint32_t at(int k) { return static_cast<uint32_t>(k < KMAX - 1 ? 2 * k : KMAX - 1 + k); }
+};
+struct PieceOfOddWorkgroup { // pieces 1, 3, ..., 2 KMAX - 3
+    static constexpr uint32_t at(int k) { return static_cast<uint32_t>(2 * k + 1); }
+};
 template <class Sum, int NSRC>
 __global__ void __launch_bounds__(kPhasedBlock)
 sum_phased_skewed_kernel(SrcTable<NSRC> src, char *out, size_t bytes, size_t tail_first, size_t numel)
 {
     constexpr int KMAX = kPhasedVecs;                                   // one vector per lane per iteration
     constexpr size_t span = static_cast<size_t>(kPhasedBlock) * kVecBytes;
-    const size_t pair_off = static_cast<size_t>(blockIdx.x >> 1) * (2 * KMAX * span);
+    constexpr size_t region = 2 * KMAX * span;
+    const size_t pair_off = static_cast<size_t>(blockIdx.x >> 1) * region;
+    const size_t left = bytes > pair_off ? bytes - pair_off : 0;
+    const uint32_t valid = static_cast<uint32_t>(left < region ? left : region);
     char *const dst[1] = {out};
-    if (blockIdx.x & 1) {
-        const size_t off = pair_off + (KMAX + 1) * span;
-        const size_t left = bytes > off ? bytes - off : 0;
-        constexpr size_t tile_bytes = (KMAX - 1) * span;
-        sum_tile_phased<Sum, NSRC, 1, 1, KMAX - 1, true, Sum::kPaceLoads>(
-            src.p, dst, off, static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes), KMAX - 1);
-    } else {
-        const size_t left = bytes > pair_off ? bytes - pair_off : 0;
-        constexpr size_t tile_bytes = (KMAX + 1) * span;
-        sum_tile_phased<Sum, NSRC, 1, 1, KMAX + 1, true, Sum::kPaceLoads>(
-            src.p, dst, pair_off, static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes), KMAX + 1);
-    }
+    if (blockIdx.x & 1)
+        sum_tile_phased<Sum, NSRC, 1, 1, KMAX - 1, true, Sum::kPaceLoads, kAuxLoadStream, PieceOfOddWorkgroup>(
+            src.p, dst, pair_off, valid, KMAX - 1);
+    else
+        sum_tile_phased<Sum, NSRC, 1, 1, KMAX + 1, true, Sum::kPaceLoads, kAuxLoadStream, PieceOfEvenWorkgroup<KMAX>>(
+            src.p, dst, pair_off, valid, KMAX + 1);
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
 }
 

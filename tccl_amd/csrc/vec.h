@@ -262,8 +262,14 @@ struct PhasedUnroll {
 // iterations of kPhasedBlock * U vectors.  valid is a multiple of 16 (may be 0).
 // FULL = the tile has exactly KMAX iterations: straight-line code, which lets the
 // compiler start the loads of the next iteration before the adds of this one.
-// LAUX = cache policy of the loads.
-template <class Sum, int NSRC, int NDST, int U, int KMAX, bool FULL, bool PACE = false, int LAUX = kAuxLoadStream>
+// LAUX = cache policy of the loads.  PIECE maps an iteration to the place of its
+// kPhasedBlock * U vectors inside the tile (in units of that many vectors): the identity
+// for a contiguous tile, something else when workgroups interleave their tiles.
+struct PieceInOrder {
+    static constexpr uint32_t at(int k) { return static_cast<uint32_t>(k); }
+};
+template <class Sum, int NSRC, int NDST, int U, int KMAX, bool FULL, bool PACE = false, int LAUX = kAuxLoadStream,
+          class PIECE = PieceInOrder>
 __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], char *const (&dst)[NDST],
                                                 size_t tile_off, uint32_t valid_bytes, int kcount)
 {
@@ -283,7 +289,7 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
 #pragma unroll
                 for (int s = 0; s < NSRC; ++s)
                     v[u][s] = __builtin_amdgcn_raw_buffer_load_b128(
-                        rs[s], k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, LAUX);
+                        rs[s], PIECE::at(k) * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, LAUX);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 Sum acc;
@@ -309,8 +315,9 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
             if (FULL || k < kcount) {
 #pragma unroll
                 for (int u = 0; u < U; ++u)
-                    __builtin_amdgcn_raw_buffer_store_b128(
-                        r[k][u], rd, k * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxStoreStream);
+                    __builtin_amdgcn_raw_buffer_store_b128(r[k][u], rd,
+                                                           PIECE::at(k) * span_bytes + u * (kPhasedBlock * kVecBytes) + lane_off,
+                                                           0, kAuxStoreStream);
             }
         }
     }
