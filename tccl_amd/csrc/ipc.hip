@@ -22,10 +22,13 @@ constexpr uint32_t kBarrierDefaultSpins = 1u << 22;
 // workgroup g raises slot g * world + rank in rank i's pad (a system-scope store: the pad
 // belongs to another process) and waits until slot g * world + i of its own pad has been
 // raised by rank i, then lowers it again, so a pad that starts zero-filled is zero-filled after
-// every completed barrier (triton_barrier.py:49-54).  One writer and one reader per slot, so
-// the reference's compare-and-swap loops are a store and a polling load.  Waits are bounded: a
-// lane that polls spin_limit times without seeing its peer sets *timeout_flag (if given) and
-// gives up; the kernel always ends.
+// every completed barrier (triton_barrier.py:49-54).  A slot has one writer of 1 (the sender)
+// and one writer of 0 (the owner), so the reference's compare-and-swap loops become "wait until
+// the slot reads 0, store 1" on the sending side and "wait until it reads 1, store 0" on the
+// receiving side.  The sender's wait matters: a rank may enter its next barrier while a peer
+// has seen, but not yet lowered, the flag of the previous one, and a flag raised then would be
+// wiped out with the old one.  Waits are bounded: a lane that polls spin_limit times in vain
+// sets *timeout_flag (if given) and gives up; the kernel always ends.
 struct PadTable {
     uint32_t *p[TCCL_MAX_WORLD];
 };
@@ -43,14 +46,30 @@ __global__ void __launch_bounds__(64) blockwise_barrier_kernel(PadTable pads, in
         if (i == lane) theirs = pad[i] + base + rank;
         if (i == rank) mine = pad[i] + base + lane;
     }
-    __hip_atomic_store(theirs, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     uint32_t polls = 0;
-    while (__hip_atomic_load(mine, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == 0u) {
+    bool expired = false;
+    // send: the slot must have been lowered by its owner since this rank last raised it
+    while (__hip_atomic_load(theirs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0u) {
         if (++polls >= spin_limit) {
-            if (timeout_flag != nullptr) __hip_atomic_store(timeout_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            return;
+            expired = true;
+            break;
         }
         __builtin_amdgcn_s_sleep(8);
+    }
+    if (!expired) {
+        __hip_atomic_store(theirs, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        // wait: the peer's flag in this rank's pad
+        while (__hip_atomic_load(mine, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == 0u) {
+            if (++polls >= spin_limit) {
+                expired = true;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(8);
+        }
+    }
+    if (expired) {
+        if (timeout_flag != nullptr) __hip_atomic_store(timeout_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        return;
     }
     __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }

@@ -60,6 +60,7 @@ class IpcWorld:
         self.lib = _lib.load()
         self._allocs: List[int] = []          # own allocations
         self._opened: List[int] = []          # peers' allocations mapped here
+        self._tables = {}                     # own buffer address -> (all ranks' addresses, bytes, dtype)
         self._count = 0
         self._host_barriers = 0
         self._flag = ctypes.POINTER(ctypes.c_uint32)()
@@ -125,7 +126,16 @@ class IpcWorld:
         ptrs = self._exchange(own, "buf")
         tensor = _as_tensor(own, nbytes, self.device).view(dtype)
         symm.register_remote(tensor, self.rank, ptrs)
+        self._tables[own] = (ptrs, nbytes, dtype)
         return tensor
+
+    def peers(self, tensor: torch.Tensor) -> List[torch.Tensor]:
+        """All ranks' buffers of the symmetric allocation ``tensor`` came from, in rank order (this
+        rank's own at index ``rank``), as tensors over the mapped memory: what the reference gets
+        from ``symm_mem.get_buffer(rank, ...)``.  Reading a peer's buffer is ordered against the
+        peer's writes by ``barrier()`` like everything else."""
+        ptrs, nbytes, dtype = self._tables[tensor.data_ptr()]
+        return [_as_tensor(p, nbytes, self.device).view(dtype) for p in ptrs]
 
     def host_barrier(self) -> None:
         """All ranks have reached this point on the host (through the directory)."""
@@ -151,6 +161,17 @@ class IpcWorld:
             self._flag[0] = 0
             raise _lib.TcclError("tccl_blockwise_barrier", _lib.TCCL_ETIMEOUT, "a peer did not reach the barrier in time")
 
+    def reset(self) -> None:
+        """Collective: bring the signal pads back to zero after a barrier wait expired (a barrier that
+        gave up leaves flags standing).  Every rank calls it; the ranks meet on the host before and
+        after, so no barrier kernel is running while the pads are cleared."""
+        torch.cuda.synchronize(self.device)
+        self.host_barrier()
+        _as_tensor(self._pad_ptrs[self.rank], self.PAD_BYTES, self.device).zero_()
+        torch.cuda.synchronize(self.device)
+        self._flag[0] = 0
+        self.host_barrier()
+
     def close(self) -> None:
         """Unmap the peers' buffers and free the own ones (after a last host barrier, so that nobody
         unmaps what a peer is still using)."""
@@ -163,6 +184,7 @@ class IpcWorld:
         for p in self._allocs:
             self.lib.tccl_symm_free(p)
         self._allocs = []
+        self._tables = {}
         if self._flag:
             self.lib.tccl_timeout_flag_destroy(self._flag)
             self._flag = ctypes.POINTER(ctypes.c_uint32)()

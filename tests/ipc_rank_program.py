@@ -29,17 +29,48 @@ def main():
     world = ipc.IpcWorld(rank, world_size, directory)
     print(f"rank {rank}: pads exchanged", flush=True)
     if mode == "missing_peer":
-        # rank 0 waits in the barrier, nobody else comes: its wait must expire and be reported
+        # rank 0 waits in the barrier, nobody else comes: its wait must expire and be reported;
+        # after a collective reset of the pads the barrier works again for everybody
+        reported = False
         if rank == 0:
             world.barrier(spin_limit=2000)
             try:
                 world.check()
             except tccl_amd.TcclError as e:
                 print(f"rank 0: reported: {e}", flush=True)
-                world.host_barrier()
-                return 42
-            return 1
-        world.host_barrier()
+                reported = True
+        world.reset()
+        for _ in range(3):
+            world.barrier()
+        world.check()
+        print(f"rank {rank}: barrier works after the reset", flush=True)
+        world.close()
+        return 42 if reported else (0 if rank != 0 else 1)
+
+    if mode == "barrier_storm":
+        # Barriers back to back with nothing but a tiny kernel between them, ranks arriving out of
+        # step: before barrier i every rank writes i into its cell, after it every rank reads all
+        # cells, and a second barrier keeps anybody from writing i + 1 before all have read i.
+        rounds = 120
+        cell = world.empty(4, torch.int32)
+        cells = world.peers(cell)
+        log = torch.zeros((rounds, world_size), dtype=torch.int32, device=cell.device)
+        for i in range(rounds):
+            if (i + rank) % 5 == 0:
+                torch.cuda._sleep(300_000 * (1 + rank % 3))
+            cell.fill_(i + 1)
+            world.barrier()
+            log[i] = torch.stack([c[0] for c in cells])
+            world.barrier()
+        world.check()
+        want = torch.arange(1, rounds + 1, dtype=torch.int32).unsqueeze(1).expand(rounds, world_size)
+        got = log.cpu()
+        world.close()
+        if not torch.equal(got, want):
+            bad = (got != want).nonzero()[0].tolist()
+            print(f"rank {rank}: round {bad[0]} read {got[bad[0]].tolist()}", flush=True)
+            return 3
+        print(f"rank {rank}: {2 * rounds} barriers in a row, every read in step", flush=True)
         return 0
 
     numel = 8 * world_size * 4099

@@ -67,9 +67,22 @@ def test_collectives_across_processes(world, tmp_path):
                                want_fp[r * perf:(r + 1) * perf].view(torch.int32)), f"round {round_} rank {r}: reduce-scatter f32"
 
 
+@pytest.mark.parametrize("world", [3, 8])
+def test_barriers_back_to_back_with_ranks_out_of_step(world, tmp_path):
+    """A rank may enter its next barrier while a peer has seen, but not yet lowered, the flag of the
+    previous one: the sender has to wait for the slot to be lowered, or its new flag is wiped out
+    with the old one.  240 barriers per rank with nothing but a tiny kernel between them, some
+    ranks delayed now and then; every read between two barriers must see that round's values."""
+    print(f"ipc: barriers back to back, {world} processes", flush=True)
+    codes, outs = run_ranks(world, tmp_path, "barrier_storm", timeout=150)
+    assert codes == [0] * world, "\n".join(outs)
+
+
 def test_barrier_with_a_missing_peer_gives_up_and_says_so(tmp_path):
     """Failure handling forced from the host: rank 0 enters the barrier with a small spin limit and
-    no peer ever does.  Its kernel must end by itself and the rank must be told."""
+    no peer ever does.  Its kernel must end by itself and the rank must be told; the flag it left
+    standing in the peer's pad is cleared by a collective reset, after which barriers work again."""
     codes, outs = run_ranks(2, tmp_path, "missing_peer", timeout=90)
     assert codes == [42, 0], "\n".join(outs)
     assert "did not reach the barrier" in outs[0]
+    assert all("barrier works after the reset" in o for o in outs)
