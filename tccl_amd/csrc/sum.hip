@@ -129,9 +129,12 @@ sum_phased_skewed_kernel(SrcTable<NSRC> src, char *out, size_t bytes, size_t tai
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
 }
 
+// Outputs up to this size take the plan for small inputs (see launch_phased).
+constexpr size_t kSmallInputBytes = static_cast<size_t>(8) << 20;
+
 template <class Sum, int NSRC, int U>
 static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t numel, const tccl_launch_cfg *cfg,
-                                  hipStream_t stream)
+                                  hipStream_t stream, bool small_input = false)
 {
     constexpr size_t kmax = kPhasedVecs / U;
     constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
@@ -141,6 +144,12 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
     size_t kcount;
     if (cfg && cfg->tile_iters > 0) {
         kcount = static_cast<size_t>(cfg->tile_iters) > kmax ? kmax : cfg->tile_iters;
+    } else if (small_input) {
+        // one launch of at most two workgroups per compute unit, with the fewest iterations that
+        // cover the input (see launch_phased)
+        kcount = (nvec + wgs * span - 1) / (wgs * span);
+        if (kcount < 1) kcount = 1;
+        if (kcount > kmax) kcount = kmax;
     } else if (NSRC <= 3 && !(cfg && cfg->grid > 0) &&
                nvec * kVecBytes >= (static_cast<size_t>(NSRC <= 2 ? 48 : 96) << 20)) {
         // With three sources or fewer a quarter or more of the traffic is writes and there
@@ -208,6 +217,23 @@ static hipError_t launch_phased(const char *const *srcs, char *out, size_t numel
 {
     if (cfg && cfg->unroll == PhasedUnroll<NSRC>::alt)
         return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::alt>(srcs, out, numel, cfg, stream);
+    if (cfg == nullptr) {
+        // Up to 8 MiB of output the launch is over before the memory system has reached its steady
+        // state, and what counts is how soon every byte has been asked for: one or two iterations
+        // per workgroup with 16 loads of 16 bytes per lane in flight (twice the usual vectors per
+        // iteration), as long as that still gives every compute unit a workgroup.  Measured on
+        // buffers rotated so that nothing is cached, against the plans for larger inputs: 8 sources
+        // 2 MiB -18 %, 4 MiB -12 %, 8 MiB -5 %; 4 sources -16 %, -8 %, -6 %; 2 sources 8 MiB -6 %;
+        // at 16 MiB the difference is gone.
+        constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
+        const size_t nvec = numel / per_vec;
+        const size_t one_per_cu = static_cast<size_t>(compute_units()) * kPhasedBlock;
+        if (nvec * kVecBytes <= kSmallInputBytes) {
+            if (nvec >= one_per_cu * PhasedUnroll<NSRC>::alt)
+                return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::alt>(srcs, out, numel, cfg, stream, true);
+            return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::value>(srcs, out, numel, cfg, stream, true);
+        }
+    }
     return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::value>(srcs, out, numel, cfg, stream);
 }
 
@@ -229,9 +255,9 @@ static hipError_t launch_phased_nsrc(const char *const *srcs, int nsrc, char *ou
 }
 
 // Inputs with at least this many output bytes take the phased kernel; smaller ones finish
-// in a few microseconds either way and take the grid-stride kernel, whose launch shape
-// adapts to tiny inputs.
-static size_t phased_min_bytes(int) { return static_cast<size_t>(4) << 20; }
+// in a few microseconds either way (the time of a launch) and take the grid-stride kernel,
+// whose launch shape adapts to tiny inputs.
+static size_t phased_min_bytes(int nsrc) { return static_cast<size_t>(nsrc <= 2 ? 4 : 2) << 20; }
 
 // Sum `nsrc` already-offset source pointers into `out`.  Shared by the three entry points.
 int sum_streams(const void *const *srcs, int nsrc, void *out, size_t numel, int dtype, hipStream_t stream,

@@ -151,11 +151,13 @@ def test_phased_and_streaming_kernels_agree_at_headline_size(_gpu_hygiene, c_ora
         assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0), cfg=cfg), want, f"flags={flags}")
 
 
-@pytest.mark.parametrize("world,mib", [(8, 4), (8, 64), (5, 64), (4, 64), (3, 96), (2, 48), (1, 48), (1, 4)])
+@pytest.mark.parametrize("world,mib", [(8, 2), (3, 2), (8, 4), (4, 4), (8, 8), (4, 8), (2, 8), (8, 64), (5, 64), (4, 64), (3, 96),
+                                       (2, 48), (1, 48), (1, 4)])
 def test_all_reduce_around_dispatch_thresholds(world, mib, _gpu_hygiene, c_oracle):
     """Sizes one vector below, at, one vector above and raggedly above every size at which
-    the library changes kernel or launch plan (grid-stride -> phased at 4 MiB of output, one
-    resident wave of tiles at 64 MiB, the single-launch rule for few sources at 48/96 MiB)."""
+    the library changes kernel or launch plan (grid-stride -> phased at 2 or 4 MiB of output, the
+    plan for small inputs up to 8 MiB and its switch to more vectors per iteration, one resident
+    wave of tiles at 64 MiB, the single-launch rule for few sources at 48/96 MiB)."""
     base = (mib << 20) // 2
     top = base + 8 * 1025 + 3
     torch.manual_seed(world * 1000 + mib)
