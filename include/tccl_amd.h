@@ -257,6 +257,23 @@ int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs,
                                           void *const *signal_pads, size_t pad_bytes, int world,
                                           size_t numel, int dtype, size_t chunk_elems,
                                           const tccl_pipeline_cfg *cfg, void *stream);
+/* The same kernel as ONE RANK's launch: the form the reference runs it in
+ * (triton_double_tree_allreduce.py:338-370, one kernel per rank, the ranks meeting through
+ * wait/send on pads in each other's memory, :175-225).  Every rank -- a process of its own on
+ * the same GPU -- makes this call with its own `rank`; bufs and signal_pads are the same tables
+ * in every rank's address space (peers' entries as opened with tccl_ipc_open), `out` is this
+ * rank's output (may be NULL).  (Ranks that share a process use the one-launch form above: the
+ * library runs a process's signalling launches one after the other, so they could never meet.)  The W launches must be able to run
+ * at the same time (each holds 1/world of the workgroups that fit the GPU) and must all be given
+ * the same numel, dtype, chunk_elems and cfg.  Between two collectives on the same buffers and
+ * pads every rank must have finished the first before any rank starts the second (and the inputs
+ * must be in place before any rank starts): tccl_blockwise_barrier() before and after, as the
+ * reference begins its kernels with blockwise_barrier.  TCCL_PIPE_DRAW_PLACES does not apply
+ * (TCCL_EINVAL).  Time-outs, pads, chunking, arithmetic: as above. */
+int tccl_double_tree_all_reduce_pipelined_rank(void *const *bufs, void *out, void *const *signal_pads,
+                                               size_t pad_bytes, int world, int rank, size_t numel,
+                                               int dtype, size_t chunk_elems,
+                                               const tccl_pipeline_cfg *cfg, void *stream);
 int tccl_signal_pad_timeouts(const void *pad0, size_t pad_bytes, unsigned *timeouts_out,
                              void *stream);
 

@@ -85,6 +85,8 @@ SIGNATURES = {
     "tccl_double_tree_signal_pad_bytes": (_SZ, [_I, _SZ, _I, _SZ]),
     "tccl_double_tree_all_reduce_pipelined": (_I, [_PP, _PP, _PP, _SZ, _I, _SZ, _I, _SZ,
                                                    ctypes.POINTER(PipelineCfg), _P]),
+    "tccl_double_tree_all_reduce_pipelined_rank": (_I, [_PP, _P, _PP, _SZ, _I, _I, _SZ, _I, _SZ,
+                                                        ctypes.POINTER(PipelineCfg), _P]),
     "tccl_signal_pad_timeouts": (_I, [_P, _SZ, ctypes.POINTER(ctypes.c_uint), _P]),
     "tccl_two_shot_all_reduce": (_I, [_PP, _PP, _PP, _SZ, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
     "tccl_two_shot_all_reduce_static": (_I, [_PP, _PP, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),

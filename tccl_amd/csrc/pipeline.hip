@@ -112,6 +112,7 @@ struct PipeArgs {
     uint32_t spin_limit;
     int world, wgs_per_rank, lag, tree_height;
     int draw;         // 1 = workgroups draw their places when they start, 0 = places follow the hardware index
+    int only_rank;    // >= 0: the launch holds this rank's workgroups only (one launch per rank); -1: all ranks'
     uint32_t *ctl;    // the control words at the end of pad 0 (place counters ... time-outs)
     uint32_t *report; // optional word in host memory that is set to 1 when a wait expires
 };
@@ -400,7 +401,14 @@ __global__ void __launch_bounds__(kPhasedBlock) tree_pipelined_kernel(PipeArgs a
     __shared__ uint32_t lds_place[2];
     int rank;
     uint32_t g;
-    take_place(a.ctl, a.draw != 0, a.world, a.wgs_per_rank, &rank, &g, lds_place);
+    if (a.only_rank >= 0) {
+        // one launch per rank (the reference's form: every rank runs its own kernel and meets the
+        // others through the pads): the grid is this rank's workgroups
+        rank = a.only_rank;
+        g = blockIdx.x;
+    } else {
+        take_place(a.ctl, a.draw != 0, a.world, a.wgs_per_rank, &rank, &g, lds_place);
+    }
     if (g != kNoPlace) tree_pipelined_walk<Sum, VECS>(a, rank, g, &lds_ok);
 }
 
@@ -467,7 +475,8 @@ static int launch_pipelined(const PipeArgs &a, int wgs_wanted, int world, size_t
     PipeArgs args = a;
     args.wgs_per_rank = per_rank;
     SignallingLaunch guard(s);
-    hipLaunchKernelGGL((tree_pipelined_kernel<Sum, VECS>), dim3(static_cast<unsigned>(per_rank * world)),
+    const int ranks_in_launch = a.only_rank >= 0 ? 1 : world;
+    hipLaunchKernelGGL((tree_pipelined_kernel<Sum, VECS>), dim3(static_cast<unsigned>(per_rank * ranks_in_launch)),
                        dim3(kPhasedBlock), 0, s, args);
     const hipError_t e = hipGetLastError();
     if (e == hipSuccess) guard.launched();
@@ -534,9 +543,12 @@ extern "C" size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int
     return (words * sizeof(uint32_t) + 15) / 16 * 16;
 }
 
-extern "C" int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs, void *const *signal_pads,
-                                                     size_t pad_bytes, int world, size_t numel, int dtype,
-                                                     size_t chunk_elems, const tccl_pipeline_cfg *cfg, void *stream)
+// Both forms of the pipelined double tree: only_rank < 0 -- one launch holding every rank's
+// workgroups, outs = W outputs or null; only_rank >= 0 -- that rank's launch, outs[only_rank]
+// its output (the other entries are not read).
+static int pipelined_double_tree(void *const *bufs, void *const *outs, void *const *signal_pads, size_t pad_bytes,
+                                 int world, int only_rank, size_t numel, int dtype, size_t chunk_elems,
+                                 const tccl_pipeline_cfg *cfg, void *stream)
 {
     if (bufs == nullptr || signal_pads == nullptr) return TCCL_EINVAL;
     PipeGeometry g;
@@ -577,7 +589,8 @@ extern "C" int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *co
     a.chunk_bytes = static_cast<uint32_t>(g.chunk_bytes);
     a.slots = static_cast<uint32_t>(g.slots);
     a.world = world;
-    a.draw = (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
+    a.only_rank = only_rank;
+    a.draw = (only_rank < 0 && cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
     a.ctl = a.pad[0] + pad_bytes / sizeof(uint32_t) - kCtlWords; // the last words of pad 0
     a.report = cfg ? cfg->timeout_flag : nullptr;
     a.spin_limit = (cfg && cfg->spin_limit > 0) ? cfg->spin_limit : kPipeDefaultSpins;
@@ -589,6 +602,26 @@ extern "C" int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *co
     const int wgs = cfg ? cfg->workgroups : 0;
     return dtype == TCCL_BF16 ? launch_pipelined_tile<Bf16Sum>(a, tile_kib, wgs, world, g.slots, s)
                               : launch_pipelined_tile<F32Sum>(a, tile_kib, wgs, world, g.slots, s);
+}
+
+extern "C" int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs, void *const *signal_pads,
+                                                     size_t pad_bytes, int world, size_t numel, int dtype,
+                                                     size_t chunk_elems, const tccl_pipeline_cfg *cfg, void *stream)
+{
+    return pipelined_double_tree(bufs, outs, signal_pads, pad_bytes, world, -1, numel, dtype, chunk_elems, cfg, stream);
+}
+
+extern "C" int tccl_double_tree_all_reduce_pipelined_rank(void *const *bufs, void *out, void *const *signal_pads,
+                                                          size_t pad_bytes, int world, int rank, size_t numel,
+                                                          int dtype, size_t chunk_elems, const tccl_pipeline_cfg *cfg,
+                                                          void *stream)
+{
+    if (rank < 0 || rank >= world || world > TCCL_MAX_WORLD) return TCCL_EINVAL;
+    if (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) return TCCL_EINVAL; // places are fixed by the rank's own launch
+    void *outs[TCCL_MAX_WORLD] = {};
+    outs[rank] = out;
+    return pipelined_double_tree(bufs, out ? outs : nullptr, signal_pads, pad_bytes, world, rank, numel, dtype,
+                                 chunk_elems, cfg, stream);
 }
 
 extern "C" int tccl_signal_pad_timeouts(const void *pad0, size_t pad_bytes, unsigned *timeouts_out, void *stream)

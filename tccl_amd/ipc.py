@@ -61,6 +61,7 @@ class IpcWorld:
         self._allocs: List[int] = []          # own allocations
         self._opened: List[int] = []          # peers' allocations mapped here
         self._tables = {}                     # own buffer address -> (all ranks' addresses, bytes, dtype)
+        self._tree_pads = {}                  # pad size -> table of all ranks' pads for the double tree
         self._count = 0
         self._host_barriers = 0
         self._flag = ctypes.POINTER(ctypes.c_uint32)()
@@ -154,12 +155,44 @@ class IpcWorld:
                                              self.BARRIER_BLOCKS, spin_limit, self._flag, stream)
         _lib.check("tccl_blockwise_barrier", rc)
 
+    def double_tree_all_reduce(self, tensor: torch.Tensor, chunk_elems: int = 0,
+                               cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+        """The reference's double-tree all-reduce as it runs it (triton_double_tree_allreduce.py:338-370):
+        this rank's own launch of the pipelined kernel, meeting the other ranks' launches through
+        wait/send on signal pads in each other's memory, between a leading and a trailing barrier.
+        Collective; the symmetric buffers are overwritten (every rank's ends up holding the sum,
+        which is also returned).  Worlds of 2, 4 and 8."""
+        ptrs, nbytes, dtype = self._tables[tensor.data_ptr()]
+        code = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype]
+        numel = tensor.numel()
+        need = self.lib.tccl_double_tree_signal_pad_bytes(self.world_size, numel, code, chunk_elems)
+        if need == 0:
+            raise ValueError("the pipelined double tree takes worlds of 2, 4 or 8 and whole 16-byte vectors")
+        key = (need,)
+        if key not in self._tree_pads:                     # collective on first use, like empty()
+            self._tree_pads[key] = _lib.ptr_array(self._exchange(self._alloc(need), "treepad"))
+        pads = self._tree_pads[key]
+        use = _lib.PipelineCfg()
+        if cfg is not None:
+            ctypes.memmove(ctypes.byref(use), ctypes.byref(cfg), ctypes.sizeof(use))
+        use.timeout_flag = self._flag
+        out = torch.empty_like(tensor)
+        stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        self.barrier()                                     # every rank's input is in place
+        rc = self.lib.tccl_double_tree_all_reduce_pipelined_rank(
+            _lib.ptr_array(ptrs), out.data_ptr(), pads, need, self.world_size, self.rank, numel, code, chunk_elems,
+            ctypes.byref(use), stream)
+        _lib.check("tccl_double_tree_all_reduce_pipelined_rank", rc)
+        self.barrier()                                     # every rank is done with buffers and pads
+        return out
+
     def check(self) -> None:
         """Synchronise and raise if a barrier wait expired (a peer never arrived)."""
         torch.cuda.synchronize(self.device)
         if self._flag[0] != 0:
             self._flag[0] = 0
-            raise _lib.TcclError("tccl_blockwise_barrier", _lib.TCCL_ETIMEOUT, "a peer did not reach the barrier in time")
+            raise _lib.TcclError("tccl_blockwise_barrier", _lib.TCCL_ETIMEOUT,
+                                 "a peer did not reach the barrier in time (or a wait inside a collective's kernel expired)")
 
     def reset(self) -> None:
         """Collective: bring the signal pads back to zero after a barrier wait expired (a barrier that

@@ -18,6 +18,12 @@ import tccl_amd                       # noqa: E402
 from tccl_amd import ipc              # noqa: E402
 
 
+# (name, elements, dtype): a few chunks with a ragged last one; enough chunks for every workgroup
+# slot of the GPU to be in use (8 MiB per buffer); fp32
+DOUBLE_TREE_SHAPES = (("small", 98_760, torch.bfloat16), ("big", 4_194_304, torch.bfloat16),
+                      ("f32", 1_048_576 + 8, torch.float32))
+
+
 def save(directory, name, rank, t):
     t = t.detach().cpu().contiguous()
     view = {2: torch.int16, 4: torch.int32, 1: torch.int8}[t.element_size()]
@@ -71,6 +77,26 @@ def main():
             print(f"rank {rank}: round {bad[0]} read {got[bad[0]].tolist()}", flush=True)
             return 3
         print(f"rank {rank}: {2 * rounds} barriers in a row, every read in step", flush=True)
+        return 0
+
+    if mode == "double_tree":
+        # one launch per rank of the pipelined double tree, ranks signalling each other through
+        # pads in each other's memory; two rounds per shape on the same buffers and pads
+        for tag, numel, dtype in DOUBLE_TREE_SHAPES:
+            t = world.empty(numel, dtype)
+            for round_ in range(2):
+                torch.manual_seed(100 * round_ + rank)
+                if dtype == torch.bfloat16:
+                    t.copy_(torch.randn(numel, dtype=dtype))
+                else:
+                    t.copy_(torch.rand(numel, dtype=dtype) * 2 - 1)
+                out = world.double_tree_all_reduce(t)
+                world.check()
+                save(directory, f"double_tree_{tag}.{round_}.out", rank, out)
+                save(directory, f"double_tree_{tag}.{round_}.buf", rank, t)
+                world.host_barrier()          # nobody refills before everybody has saved
+            print(f"rank {rank}: double tree {tag} done", flush=True)
+        world.close()
         return 0
 
     numel = 8 * world_size * 4099

@@ -104,6 +104,15 @@ def test_argument_checks_return_codes_without_launching():
     assert piped(null, None, pads, 4096, 2, 64, 0, 0, None, None) == -1
     assert piped(odd, None, pads, 4096, 2, 64, 0, 0, None, None) == -2
     assert piped(good, None, pads, 4096, 2, 0, 0, 0, None, None) == 0
+    ranked = lib.tccl_double_tree_all_reduce_pipelined_rank
+    assert ranked(good, None, pads, 4096, 2, 2, 64, 0, 0, None, None) == -1   # rank outside the world
+    assert ranked(good, None, pads, 4096, 2, -1, 64, 0, 0, None, None) == -1
+    assert ranked(good, None, pads, 4096, 3, 1, 64, 0, 0, None, None) == -3
+    assert ranked(good, None, pads, 4096, 2, 1, 60, 0, 0, None, None) == -2
+    assert ranked(good, None, pads, 0, 2, 1, 64, 0, 0, None, None) == -1
+    drawn = _lib.PipelineCfg(flags=_lib.PIPE_DRAW_PLACES)
+    assert ranked(good, None, pads, 4096, 2, 1, 64, 0, 0, ctypes.byref(drawn), None) == -1   # no drawn places per rank
+    assert ranked(good, None, pads, 4096, 2, 1, 0, 0, 0, None, None) == 0
     two = lib.tccl_two_shot_all_reduce
     assert two(good, None, pads, 4096, 0, 64, 0, None, None) == -1
     assert two(good, None, pads, 4096, 9, 64, 0, None, None) == -1

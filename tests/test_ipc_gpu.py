@@ -67,6 +67,28 @@ def test_collectives_across_processes(world, tmp_path):
                                want_fp[r * perf:(r + 1) * perf].view(torch.int32)), f"round {round_} rank {r}: reduce-scatter f32"
 
 
+@pytest.mark.parametrize("world", [4, 8])
+def test_double_tree_one_launch_per_rank(world, tmp_path):
+    """The reference's double-tree design as it runs it: every rank (a process) launches its own
+    kernel, and the kernels hand chunks to each other through wait/send on pads in each other's
+    memory (triton_double_tree_allreduce.py:175-225, :338-370).  Outputs and the buffers (the
+    collective works in place) against the oracle, bit for bit, two rounds per shape."""
+    from ipc_rank_program import DOUBLE_TREE_SHAPES
+    print(f"ipc: double tree, {world} processes", flush=True)
+    codes, outs = run_ranks(world, tmp_path, "double_tree", timeout=150)
+    assert codes == [0] * world, "\n".join(outs)
+    for tag, numel, dtype in DOUBLE_TREE_SHAPES:
+        bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+        for round_ in range(2):
+            bufs = (seeded_randn(world, numel, seed_base=100 * round_) if dtype == torch.bfloat16
+                    else seeded_uniform(world, numel, seed_base=100 * round_))
+            want = torch_ref.double_tree_all_reduce(bufs)[0].view(bits)
+            for r in range(world):
+                for what in ("out", "buf"):
+                    got = load(tmp_path, f"double_tree_{tag}.{round_}.{what}", r, dtype).view(bits)
+                    assert torch.equal(got, want), f"{tag} round {round_} rank {r} {what}"
+
+
 @pytest.mark.parametrize("world", [3, 8])
 def test_barriers_back_to_back_with_ranks_out_of_step(world, tmp_path):
     """A rank may enter its next barrier while a peer has seen, but not yet lowered, the flag of the
