@@ -294,6 +294,15 @@ int tccl_signal_pad_timeouts(const void *pad0, size_t pad_bytes, unsigned *timeo
 int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *signal_pads,
                              size_t pad_bytes, int world, size_t numel, int dtype,
                              const tccl_pipeline_cfg *cfg, void *stream);
+/* The same kernel as ONE RANK's launch, for ranks that are processes of their own on the same
+ * GPU (see tccl_double_tree_all_reduce_pipelined_rank for the calling rules: same arguments in
+ * every rank, the W launches running at the same time, tccl_blockwise_barrier() before and
+ * after).  The barrier between the two shots is then exactly the reference's construct: a
+ * blockwise barrier between kernels of different owners (triton_barrier.py:39-142), inside the
+ * kernel.  `out` = this rank's output or NULL (the result is in bufs[rank] either way). */
+int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void *const *signal_pads,
+                                  size_t pad_bytes, int world, int rank, size_t numel, int dtype,
+                                  const tccl_pipeline_cfg *cfg, void *stream);
 
 /* tccl_two_shot_all_reduce() for callers that cannot allocate the signal pads it needs -- code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no

@@ -648,6 +648,7 @@ struct TwoShotArgs {
     uint32_t spin_limit;
     int world, wgs_per_rank;
     int draw;         // 1 = workgroups draw their places when they start, 0 = places follow the hardware index
+    int only_rank;    // >= 0: the launch holds this rank's workgroups only (one launch per rank); -1: all ranks'
     uint32_t *ctl;    // control words at the end of pad 0 (place counters ... time-outs)
     uint32_t *report; // optional host word set to 1 when a wait expires
 };
@@ -766,7 +767,14 @@ __global__ void __launch_bounds__(kPhasedBlock) two_shot_kernel(TwoShotArgs a)
     __shared__ uint32_t lds_place[2];
     int rank;
     uint32_t g;
-    take_place(a.ctl, a.draw != 0, W, a.wgs_per_rank, &rank, &g, lds_place);
+    if (a.only_rank >= 0) {
+        // one launch per rank: the barrier between the shots is then the reference's own
+        // construct, a barrier between the kernels of different owners
+        rank = a.only_rank;
+        g = blockIdx.x;
+    } else {
+        take_place(a.ctl, a.draw != 0, W, a.wgs_per_rank, &rank, &g, lds_place);
+    }
     if (g != kNoPlace) two_shot_body<Sum, W>(a, rank, g, lds_ok);
 }
 
@@ -829,8 +837,9 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, cons
         const hipError_t ce = hipGetLastError();
         if (ce != hipSuccess) return hip_code(ce);
     }
-    hipLaunchKernelGGL((two_shot_kernel<Sum, W>), dim3(static_cast<unsigned>(per_rank * W)), dim3(kPhasedBlock), 0, s,
-                       a);
+    const size_t ranks_in_launch = a.only_rank >= 0 ? 1 : W;
+    hipLaunchKernelGGL((two_shot_kernel<Sum, W>), dim3(static_cast<unsigned>(per_rank * ranks_in_launch)),
+                       dim3(kPhasedBlock), 0, s, a);
     const hipError_t e = hipGetLastError();
     if (e == hipSuccess) guard.launched();
     return hip_code(e);
@@ -872,7 +881,8 @@ static int two_shot_check(void *const *bufs, void *const *outs, int world, size_
 
 // The launch itself: `pads` are the W signal pads (device addresses), each of pad_bytes.
 static int two_shot_launch(void *const *bufs, void *const *outs, uint32_t *const *pads, size_t pad_bytes, int world,
-                           size_t numel, int dtype, const tccl_pipeline_cfg *cfg, const ClearRequest *clear, hipStream_t s)
+                           size_t numel, int dtype, const tccl_pipeline_cfg *cfg, const ClearRequest *clear, hipStream_t s,
+                           int only_rank = -1)
 {
     TwoShotArgs a = {};
     for (int r = 0; r < world; ++r) {
@@ -886,7 +896,8 @@ static int two_shot_launch(void *const *bufs, void *const *outs, uint32_t *const
     const size_t pad_words = pad_bytes / sizeof(uint32_t);
     a.ctl = a.pad[0] + pad_words - kCtlWords;
     a.report = cfg ? cfg->timeout_flag : nullptr;
-    a.draw = (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
+    a.only_rank = only_rank;
+    a.draw = (only_rank < 0 && cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
     const int wgs = cfg ? cfg->workgroups : 0;
     return dtype == TCCL_BF16 ? launch_two_shot_world<Bf16Sum>(a, wgs, pad_words, clear, s)
                               : launch_two_shot_world<F32Sum>(a, wgs, pad_words, clear, s);
@@ -913,6 +924,30 @@ extern "C" int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, vo
     if (nothing) return TCCL_OK;
     return two_shot_launch(bufs, outs, pads, pad_bytes, world, numel, dtype, cfg, nullptr,
                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes,
+                                             int world, int rank, size_t numel, int dtype,
+                                             const tccl_pipeline_cfg *cfg, void *stream)
+{
+    if (signal_pads == nullptr || world < 1 || world > TCCL_MAX_WORLD || rank < 0 || rank >= world) return TCCL_EINVAL;
+    if (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) return TCCL_EINVAL; // places are fixed by the rank's own launch
+    if (pad_bytes % 16 != 0 || pad_bytes < (static_cast<size_t>(world) + kCtlWords) * sizeof(uint32_t))
+        return TCCL_EINVAL;
+    void *outs[TCCL_MAX_WORLD] = {};
+    outs[rank] = out;
+    bool nothing = false;
+    const int rc = two_shot_check(bufs, out ? outs : nullptr, world, numel, dtype, &nothing);
+    if (rc != TCCL_OK) return rc;
+    uint32_t *pads[TCCL_MAX_WORLD];
+    for (int r = 0; r < world; ++r) {
+        if (signal_pads[r] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(signal_pads[r])) return TCCL_EALIGN;
+        pads[r] = static_cast<uint32_t *>(signal_pads[r]);
+    }
+    if (nothing) return TCCL_OK;
+    return two_shot_launch(bufs, out ? outs : nullptr, pads, pad_bytes, world, numel, dtype, cfg, nullptr,
+                           static_cast<hipStream_t>(stream), rank);
 }
 
 // ------------------------------------------------------------------ the entry point that allocates nothing

@@ -61,7 +61,7 @@ class IpcWorld:
         self._allocs: List[int] = []          # own allocations
         self._opened: List[int] = []          # peers' allocations mapped here
         self._tables = {}                     # own buffer address -> (all ranks' addresses, bytes, dtype)
-        self._tree_pads = {}                  # pad size -> table of all ranks' pads for the double tree
+        self._tree_pads = {}                  # pad size -> table of all ranks' pads for kernels that signal inside a launch
         self._count = 0
         self._host_barriers = 0
         self._flag = ctypes.POINTER(ctypes.c_uint32)()
@@ -155,23 +155,20 @@ class IpcWorld:
                                              self.BARRIER_BLOCKS, spin_limit, self._flag, stream)
         _lib.check("tccl_blockwise_barrier", rc)
 
-    def double_tree_all_reduce(self, tensor: torch.Tensor, chunk_elems: int = 0,
-                               cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
-        """The reference's double-tree all-reduce as it runs it (triton_double_tree_allreduce.py:338-370):
-        this rank's own launch of the pipelined kernel, meeting the other ranks' launches through
-        wait/send on signal pads in each other's memory, between a leading and a trailing barrier.
-        Collective; the symmetric buffers are overwritten (every rank's ends up holding the sum,
-        which is also returned).  Worlds of 2, 4 and 8."""
-        ptrs, nbytes, dtype = self._tables[tensor.data_ptr()]
+    # Signal pad size the two-shot kernel is given: room for 1024 workgroups per rank.
+    TWO_SHOT_PAD_BYTES = 4 * (8 * 1024 + 288)
+
+    def _kernel_pads(self, nbytes: int) -> ctypes.Array:
+        """All ranks' signal pads of `nbytes` for the kernels that signal inside a launch (collective on
+        first use of a size, like ``empty``)."""
+        if nbytes not in self._tree_pads:
+            self._tree_pads[nbytes] = _lib.ptr_array(self._exchange(self._alloc(nbytes), "kpad"))
+        return self._tree_pads[nbytes]
+
+    def _own_launch(self, name: str, tensor: torch.Tensor, pad_bytes: int, tail_args, cfg) -> torch.Tensor:
+        ptrs, _, dtype = self._tables[tensor.data_ptr()]
         code = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype]
-        numel = tensor.numel()
-        need = self.lib.tccl_double_tree_signal_pad_bytes(self.world_size, numel, code, chunk_elems)
-        if need == 0:
-            raise ValueError("the pipelined double tree takes worlds of 2, 4 or 8 and whole 16-byte vectors")
-        key = (need,)
-        if key not in self._tree_pads:                     # collective on first use, like empty()
-            self._tree_pads[key] = _lib.ptr_array(self._exchange(self._alloc(need), "treepad"))
-        pads = self._tree_pads[key]
+        pads = self._kernel_pads(pad_bytes)
         use = _lib.PipelineCfg()
         if cfg is not None:
             ctypes.memmove(ctypes.byref(use), ctypes.byref(cfg), ctypes.sizeof(use))
@@ -179,12 +176,33 @@ class IpcWorld:
         out = torch.empty_like(tensor)
         stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
         self.barrier()                                     # every rank's input is in place
-        rc = self.lib.tccl_double_tree_all_reduce_pipelined_rank(
-            _lib.ptr_array(ptrs), out.data_ptr(), pads, need, self.world_size, self.rank, numel, code, chunk_elems,
-            ctypes.byref(use), stream)
-        _lib.check("tccl_double_tree_all_reduce_pipelined_rank", rc)
+        rc = getattr(self.lib, name)(_lib.ptr_array(ptrs), out.data_ptr(), pads, pad_bytes, self.world_size, self.rank,
+                                     tensor.numel(), code, *tail_args, ctypes.byref(use), stream)
+        _lib.check(name, rc)
         self.barrier()                                     # every rank is done with buffers and pads
         return out
+
+    def double_tree_all_reduce(self, tensor: torch.Tensor, chunk_elems: int = 0,
+                               cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+        """The reference's double-tree all-reduce as it runs it (triton_double_tree_allreduce.py:338-370):
+        this rank's own launch of the pipelined kernel, meeting the other ranks' launches through
+        wait/send on signal pads in each other's memory, between a leading and a trailing barrier.
+        Collective; the symmetric buffers are overwritten (every rank's ends up holding the sum,
+        which is also returned).  Worlds of 2, 4 and 8."""
+        _, _, dtype = self._tables[tensor.data_ptr()]
+        code = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype]
+        need = self.lib.tccl_double_tree_signal_pad_bytes(self.world_size, tensor.numel(), code, chunk_elems)
+        if need == 0:
+            raise ValueError("the pipelined double tree takes worlds of 2, 4 or 8 and whole 16-byte vectors")
+        return self._own_launch("tccl_double_tree_all_reduce_pipelined_rank", tensor, need, (chunk_elems,), cfg)
+
+    def two_shot_all_reduce(self, tensor: torch.Tensor, cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+        """Two-shot all-reduce, this rank's own launch: reduce the own share from all buffers, meet
+        the other ranks' kernels in the reference's blockwise barrier (triton_barrier.py:39-142,
+        inside the kernel, as the reference uses it), gather the other shares.  Collective, in
+        place (every buffer ends up holding the sum, which is also returned); bit-identical to
+        ``one_shot_all_reduce``.  The element count must be a multiple of W vectors."""
+        return self._own_launch("tccl_two_shot_all_reduce_rank", tensor, self.TWO_SHOT_PAD_BYTES, (), cfg)
 
     def check(self) -> None:
         """Synchronise and raise if a barrier wait expired (a peer never arrived)."""

@@ -24,6 +24,10 @@ DOUBLE_TREE_SHAPES = (("small", 98_760, torch.bfloat16), ("big", 4_194_304, torc
                       ("f32", 1_048_576 + 8, torch.float32))
 
 
+# (name, elements per rank's share, dtype): less than a tile; many tiles with a ragged last one; fp32
+TWO_SHOT_SHAPES = (("small", 8 * 37, torch.bfloat16), ("big", 8 * 65_537, torch.bfloat16), ("f32", 4 * 20_011, torch.float32))
+
+
 def save(directory, name, rank, t):
     t = t.detach().cpu().contiguous()
     view = {2: torch.int16, 4: torch.int32, 1: torch.int8}[t.element_size()]
@@ -96,6 +100,27 @@ def main():
                 save(directory, f"double_tree_{tag}.{round_}.buf", rank, t)
                 world.host_barrier()          # nobody refills before everybody has saved
             print(f"rank {rank}: double tree {tag} done", flush=True)
+        world.close()
+        return 0
+
+    if mode == "two_shot":
+        # one launch per rank of the two-shot kernel: the blockwise barrier between its shots is a
+        # barrier between kernels of different owners
+        for tag, numel, dtype in TWO_SHOT_SHAPES:
+            numel *= world_size
+            t = world.empty(numel, dtype)
+            for round_ in range(2):
+                torch.manual_seed(100 * round_ + rank)
+                if dtype == torch.bfloat16:
+                    t.copy_(torch.randn(numel, dtype=dtype))
+                else:
+                    t.copy_(torch.rand(numel, dtype=dtype) * 2 - 1)
+                out = world.two_shot_all_reduce(t)
+                world.check()
+                save(directory, f"two_shot_{tag}.{round_}.out", rank, out)
+                save(directory, f"two_shot_{tag}.{round_}.buf", rank, t)
+                world.host_barrier()
+            print(f"rank {rank}: two-shot {tag} done", flush=True)
         world.close()
         return 0
 

@@ -122,6 +122,13 @@ def test_argument_checks_return_codes_without_launching():
     assert two(good, None, pads, 4090, 2, 64, 0, None, None) == -1            # pad size not a multiple of 16
     assert two(null, None, pads, 4096, 2, 64, 0, None, None) == -1
     assert two(good, None, pads, 4096, 2, 0, 0, None, None) == 0
+    two_r = lib.tccl_two_shot_all_reduce_rank
+    assert two_r(good, None, pads, 4096, 2, 2, 64, 0, None, None) == -1       # rank outside the world
+    assert two_r(good, None, pads, 4096, 9, 0, 64, 0, None, None) == -1
+    assert two_r(good, None, pads, 4096, 2, 1, 24, 0, None, None) == -2
+    assert two_r(good, None, pads, 1152, 2, 1, 64, 0, None, None) == -1
+    assert two_r(good, None, pads, 4096, 2, 1, 64, 0, ctypes.byref(drawn), None) == -1
+    assert two_r(good, None, pads, 4096, 2, 1, 0, 0, None, None) == 0
     static = lib.tccl_two_shot_all_reduce_static
     assert static(good, None, 0, 64, 0, None, None) == -1
     assert static(good, None, 9, 64, 0, None, None) == -1

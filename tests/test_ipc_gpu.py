@@ -90,6 +90,29 @@ def test_double_tree_one_launch_per_rank(world, tmp_path):
 
 
 @pytest.mark.parametrize("world", [3, 8])
+def test_two_shot_one_launch_per_rank(world, tmp_path):
+    """Two-shot all-reduce with every rank (a process) launching its own kernel: the blockwise
+    barrier between the shots is then the reference's construct, a barrier between kernels of
+    different owners inside the kernel (triton_barrier.py:39-142).  Outputs and buffers against
+    the oracle's all-reduce, bit for bit, two rounds per shape."""
+    from ipc_rank_program import TWO_SHOT_SHAPES
+    print(f"ipc: two-shot, {world} processes", flush=True)
+    codes, outs = run_ranks(world, tmp_path, "two_shot", timeout=150)
+    assert codes == [0] * world, "\n".join(outs)
+    for tag, per_rank, dtype in TWO_SHOT_SHAPES:
+        numel = per_rank * world
+        bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+        for round_ in range(2):
+            bufs = (seeded_randn(world, numel, seed_base=100 * round_) if dtype == torch.bfloat16
+                    else seeded_uniform(world, numel, seed_base=100 * round_))
+            want = torch_ref.all_reduce(bufs).view(bits)
+            for r in range(world):
+                for what in ("out", "buf"):
+                    got = load(tmp_path, f"two_shot_{tag}.{round_}.{what}", r, dtype).view(bits)
+                    assert torch.equal(got, want), f"{tag} round {round_} rank {r} {what}"
+
+
+@pytest.mark.parametrize("world", [3, 8])
 def test_barriers_back_to_back_with_ranks_out_of_step(world, tmp_path):
     """A rank may enter its next barrier while a peer has seen, but not yet lowered, the flag of the
     previous one: the sender has to wait for the slot to be lowered, or its new flag is wiped out
