@@ -17,7 +17,7 @@ from typing import List, Optional
 import torch
 
 from . import _lib, spmd
-from .symm import SymmGroup, SymmHandle, rendezvous
+from .symm import SymmGroup, rendezvous
 
 _SUM_DTYPES = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}
 

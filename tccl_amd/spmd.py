@@ -18,7 +18,7 @@ W ranks have entered it, i.e. until everything they did before has been enqueued
 from __future__ import annotations
 
 import threading
-from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
+from typing import Any, Callable, Dict, List, Optional
 
 import torch
 

@@ -5,7 +5,6 @@ import os
 import re
 
 import pytest
-import torch
 
 import tccl_amd
 from tccl_amd import _lib

@@ -7,7 +7,7 @@ import torch
 
 import tccl_amd
 from tccl_amd import spmd
-from helpers import assert_bit_equal, from_np_bits, np_bits
+from helpers import assert_bit_equal
 from oracle import torch_ref
 
 pytestmark = pytest.mark.gpu
