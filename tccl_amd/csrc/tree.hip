@@ -529,26 +529,26 @@ extern "C" int tccl_double_tree_plan_create(void *const *bufs, void *const *outs
     if (e != hipSuccess) return hip_code(e);
     e = hipStreamBeginCapture(cap, hipStreamCaptureModeRelaxed);
     if (e != hipSuccess) {
-        hipStreamDestroy(cap);
+        (void)hipStreamDestroy(cap);
         return hip_code(e);
     }
     const int rc = tccl_double_tree_all_reduce(bufs, outs, world, numel, dtype, chunk_elems, cap);
     hipGraph_t graph = nullptr;
     e = hipStreamEndCapture(cap, &graph); // always end the capture, also after an argument error
-    hipStreamDestroy(cap);
+    (void)hipStreamDestroy(cap);
     if (rc != TCCL_OK || e != hipSuccess || graph == nullptr) {
-        if (graph) hipGraphDestroy(graph);
+        if (graph) (void)hipGraphDestroy(graph);
         return rc != TCCL_OK ? rc : (e != hipSuccess ? hip_code(e) : TCCL_EINVAL);
     }
     tccl_plan *plan = new (std::nothrow) tccl_plan;
     if (plan == nullptr) {
-        hipGraphDestroy(graph);
+        (void)hipGraphDestroy(graph);
         return hip_code(hipErrorOutOfMemory);
     }
     plan->graph = graph;
     e = hipGraphInstantiate(&plan->exec, graph, nullptr, nullptr, 0);
     if (e != hipSuccess) {
-        hipGraphDestroy(graph);
+        (void)hipGraphDestroy(graph);
         delete plan;
         return hip_code(e);
     }
