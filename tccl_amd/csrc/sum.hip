@@ -92,7 +92,7 @@ sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
 }
 
-// The same launch with unequal, interleaved tiles: workgroups 2p and 2p+1 share a region of
+// The same launch with unequal, interleaved tiles (three sources or more): workgroups 2p and 2p+1 share a region of
 // 2 * KMAX pieces (a piece = what one iteration covers, 4 KiB), the even one taking KMAX + 1 and
 // the odd one KMAX - 1 of them.  Workgroup b runs on XCD b mod 8, and on MI355X the odd XCDs read
 // more slowly than the even ones when the whole GPU streams from memory (their L2s wait three
@@ -127,6 +127,20 @@ sum_phased_skewed_kernel(SrcTable<NSRC> src, char *out, size_t bytes, size_t tai
         sum_tile_phased<Sum, NSRC, 1, 1, KMAX + 1, true, Sum::kPaceLoads, kAuxLoadStream, PieceOfEvenWorkgroup<KMAX>>(
             src.p, dst, pair_off, valid, KMAX + 1);
     if (blockIdx.x == 0 && tail_first < numel) sum_tail<Sum, NSRC, 1>(src.p, dst, tail_first, numel);
+}
+
+// Would the plan for one vector per lane per iteration cut `nvec` vectors into full 128 KiB
+// tiles (launch_phased_u's default rule: one or two workgroups per compute unit, fewest
+// launches, smallest tile that covers a launch's share)?
+static bool plans_full_tiles(size_t nvec)
+{
+    constexpr size_t tile = static_cast<size_t>(kPhasedBlock) * kPhasedVecs;
+    size_t wgs = static_cast<size_t>(compute_units()) * 2;
+    if (nvec <= (wgs / 2) * tile) wgs /= 2;
+    size_t launches = (nvec + wgs * tile - 1) / (wgs * tile);
+    if (launches == 0) launches = 1;
+    const size_t per_launch = (nvec + launches - 1) / launches;
+    return (per_launch + wgs * kPhasedBlock - 1) / (wgs * kPhasedBlock) >= kPhasedVecs;
 }
 
 // Outputs up to this size take the plan for small inputs (see launch_phased).
@@ -177,7 +191,7 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
     const size_t slice_vec = wgs * tile_vec;
     // full-size tiles of many sources, launch shape left to the library: unequal tiles for even and
     // odd XCDs (see sum_phased_skewed_kernel)
-    const bool skewed = U == 1 && NSRC >= 5 && kcount == kmax && cfg == nullptr && wgs % 2 == 0;
+    const bool skewed = U == 1 && NSRC >= 3 && kcount == kmax && cfg == nullptr && wgs % 2 == 0;
     const size_t tail_first = nvec * per_vec;
 
     size_t off = 0;
@@ -192,7 +206,7 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
         const size_t rel_first = last ? tail_first - off * per_vec : 0;
         const size_t rel_numel = last ? numel - off * per_vec : 0;
         if (skewed) {
-            if constexpr (U == 1 && NSRC >= 5)
+            if constexpr (U == 1 && NSRC >= 3)
                 hipLaunchKernelGGL((sum_phased_skewed_kernel<Sum, NSRC>), dim3(static_cast<unsigned>((grid + 1) / 2 * 2)),
                                    dim3(kPhasedBlock), 0, stream, t, out + off * kVecBytes, n * kVecBytes, rel_first,
                                    rel_numel);
@@ -233,6 +247,16 @@ static hipError_t launch_phased(const char *const *srcs, char *out, size_t numel
                 return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::alt>(srcs, out, numel, cfg, stream, true);
             return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::value>(srcs, out, numel, cfg, stream, true);
         }
+    }
+    if constexpr (NSRC == 3 || NSRC == 4) {
+        // Three and four sources run two vectors per iteration, except where the input is cut
+        // into full tiles: there the unequal, interleaved tiles of sum_phased_skewed_kernel (one
+        // vector per iteration) measured 2-4 % faster on rotated buffers.
+        constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
+        const size_t nvec = numel / per_vec;
+        const bool many_small_tiles = NSRC <= 3 && nvec * kVecBytes >= (static_cast<size_t>(96) << 20);
+        if (cfg == nullptr && !many_small_tiles && plans_full_tiles(nvec))
+            return launch_phased_u<Sum, NSRC, 1>(srcs, out, numel, cfg, stream);
     }
     return launch_phased_u<Sum, NSRC, PhasedUnroll<NSRC>::value>(srcs, out, numel, cfg, stream);
 }
