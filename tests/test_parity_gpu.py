@@ -151,13 +151,14 @@ def test_phased_and_streaming_kernels_agree_at_headline_size(_gpu_hygiene, c_ora
         assert_bit_equal(tccl_amd.one_shot_all_reduce(g.tensor(0), cfg=cfg), want, f"flags={flags}")
 
 
-@pytest.mark.parametrize("world,mib", [(8, 2), (3, 2), (8, 4), (4, 4), (8, 8), (4, 8), (2, 8), (8, 64), (5, 64), (4, 64), (3, 96),
-                                       (2, 48), (1, 48), (1, 4)])
+@pytest.mark.parametrize("world,mib", [(8, 2), (3, 2), (8, 4), (4, 4), (8, 8), (4, 8), (2, 8), (8, 32), (4, 32), (3, 32), (8, 64),
+                                       (5, 64), (4, 64), (3, 64), (3, 96), (2, 48), (1, 48), (1, 4)])
 def test_all_reduce_around_dispatch_thresholds(world, mib, _gpu_hygiene, c_oracle):
     """Sizes one vector below, at, one vector above and raggedly above every size at which
     the library changes kernel or launch plan (grid-stride -> phased at 2 or 4 MiB of output, the
-    plan for small inputs up to 8 MiB and its switch to more vectors per iteration, one resident
-    wave of tiles at 64 MiB, the single-launch rule for few sources at 48/96 MiB)."""
+    plan for small inputs up to 8 MiB and its switch to more vectors per iteration, full tiles
+    -- and with them unequal, interleaved tiles -- for one workgroup per compute unit at 32 MiB
+    and for two at 64 MiB, the single-launch rule for few sources at 48/96 MiB)."""
     base = (mib << 20) // 2
     top = base + 8 * 1025 + 3
     torch.manual_seed(world * 1000 + mib)
@@ -169,6 +170,24 @@ def test_all_reduce_around_dispatch_thresholds(world, mib, _gpu_hygiene, c_oracl
     for numel in (base - 8, base, base + 8, base + 8 * 1025 + 3):
         out.fill_(9.0)
         assert lib.tccl_all_reduce_sum(g.ptr_array, world, out.data_ptr(), numel, _lib.TCCL_BF16, stream()) == 0
+        want = oracle_sum(c_oracle, [b[:numel].contiguous() for b in bufs])
+        assert_bit_equal(out[:numel], want, f"W={world} numel={numel}")
+        assert out[numel:numel + 64].eq(9.0).all().item(), "wrote past the end"
+
+
+@pytest.mark.parametrize("world", [3, 4, 8])
+def test_all_reduce_f32_full_tiles(world, _gpu_hygiene, c_oracle):
+    """fp32 where the input is cut into full tiles (unequal, interleaved tiles for three sources
+    or more): exactly one wave of tiles, one element less, and a ragged size above it."""
+    base = (64 << 20) // 4
+    top = base + 4 * 1025 + 3
+    bufs = seeded_uniform(world, top, seed_base=40 + world)
+    g = upload(_gpu_hygiene, bufs)
+    lib = tccl_amd.load_library()
+    out = torch.empty(top + 64, dtype=torch.float32, device=DEV)
+    for numel in (base - 1, base, top):
+        out.fill_(9.0)
+        assert lib.tccl_all_reduce_sum(g.ptr_array, world, out.data_ptr(), numel, _lib.TCCL_F32, stream()) == 0
         want = oracle_sum(c_oracle, [b[:numel].contiguous() for b in bufs])
         assert_bit_equal(out[:numel], want, f"W={world} numel={numel}")
         assert out[numel:numel + 64].eq(9.0).all().item(), "wrote past the end"
