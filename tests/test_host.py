@@ -54,7 +54,7 @@ def test_wrapper_preconditions_match_the_reference():
     g = make_group(4, 64, torch.bfloat16)
     t = g.tensor(0)
     with pytest.raises(AssertionError, match="128-bit aligned"):
-        tccl_amd.one_shot_all_reduce(t[:12])
+        tccl_amd.one_shot_all_reduce(t[:10])            # the reference's bound here is 4 elements (:70, :74)
     with pytest.raises(AssertionError, match="128-bit aligned"):
         tccl_amd.one_shot_reduce_scatter(t[:40])        # 40 % (8*4) != 0
     with pytest.raises(AssertionError, match="128-bit aligned"):

@@ -175,6 +175,16 @@ def test_all_reduce_around_dispatch_thresholds(world, mib, _gpu_hygiene, c_oracl
         assert out[numel:numel + 64].eq(9.0).all().item(), "wrote past the end"
 
 
+def test_all_reduce_wrapper_takes_multiples_of_four_elements(_gpu_hygiene, c_oracle):
+    """The reference's wrapper accepts any multiple of 4 bf16 elements
+    (triton_one_shot_all_reduce_no_128.py:70-76), not only whole 16-byte vectors."""
+    bufs = seeded_randn(8, 8 * 1000 + 4)
+    g = upload(_gpu_hygiene, bufs)
+    for numel in (4, 12, 8 * 1000 + 4):
+        got = tccl_amd.one_shot_all_reduce(g.tensor(0)[:numel])
+        assert_bit_equal(got, oracle_sum(c_oracle, [b[:numel].contiguous() for b in bufs]), f"numel={numel}")
+
+
 @pytest.mark.parametrize("world", [3, 4, 8])
 def test_all_reduce_f32_full_tiles(world, _gpu_hygiene, c_oracle):
     """fp32 where the input is cut into full tiles (unequal, interleaved tiles for three sources

@@ -61,8 +61,8 @@ def test_a_failing_rank_releases_the_others():
 
 def test_precondition_failure_inside_a_collective_propagates():
     def main(rank, world_size):
-        t = spmd.empty_strided_p2p((12,), (1,), torch.bfloat16, "cpu")
-        return tccl_amd.one_shot_all_reduce(t)          # 12 elements: not 128-bit aligned
+        t = spmd.empty_strided_p2p((10,), (1,), torch.bfloat16, "cpu")
+        return tccl_amd.one_shot_all_reduce(t)          # 10 elements: not a multiple of the reference's 4
 
     with pytest.raises(AssertionError, match="128-bit aligned"):
         spmd.run(2, main)
