@@ -146,14 +146,21 @@ class IpcWorld:
         for r in range(self.world_size):
             self._wait_for(os.path.join(self.directory, f"{tag}.rank{r}"))
 
-    def barrier(self, spin_limit: int = 0) -> None:
+    def barrier(self, spin_limit: int = 0, blocks: Optional[int] = None) -> None:
         """The reference's ``blockwise_barrier`` on torch's current stream: everything this rank
         enqueued before is complete before any rank's later work starts.  Asynchronous; a wait
-        that expires is reported by ``check()``."""
+        that expires is reported by ``check()``.  ``blocks``: rows of slots used (the reference's
+        own test launches 32, triton_barrier.py:155-160); every rank must pass the same."""
         stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
         rc = self.lib.tccl_blockwise_barrier(self._pad_array, self.PAD_BYTES, self.world_size, self.rank,
-                                             self.BARRIER_BLOCKS, spin_limit, self._flag, stream)
+                                             self.BARRIER_BLOCKS if blocks is None else blocks, spin_limit, self._flag,
+                                             stream)
         _lib.check("tccl_blockwise_barrier", rc)
+
+    def signal_pad(self) -> torch.Tensor:
+        """This rank's signal pad as a tensor of 32-bit words (what the reference prints after its
+        barrier test, triton_barrier.py:178-190): all zero whenever no barrier is running."""
+        return _as_tensor(self._pad_ptrs[self.rank], self.PAD_BYTES, self.device).view(torch.int32)
 
     # Signal pad size the two-shot kernel is given: room for 1024 workgroups per rank.
     TWO_SHOT_PAD_BYTES = 4 * (8 * 1024 + 288)

@@ -57,6 +57,20 @@ def main():
         world.close()
         return 42 if reported else (0 if rank != 0 else 1)
 
+    if mode == "barrier_test":
+        # the reference's own barrier test (triton_barrier.py:155-190): 32 blocks per rank, one
+        # launch per rank, then look at the pad -- which must be all zero again
+        for _ in range(3):
+            world.barrier(blocks=32)
+        world.check()
+        pad = world.signal_pad().cpu()
+        world.close()
+        if int(pad.ne(0).sum()) != 0:
+            print(f"rank {rank}: pad not zero after the barrier: {pad.nonzero().flatten().tolist()[:8]}", flush=True)
+            return 4
+        print(f"rank {rank}: barrier test passed, pad is zero", flush=True)
+        return 0
+
     if mode == "barrier_storm":
         # Barriers back to back with nothing but a tiny kernel between them, ranks arriving out of
         # step: before barrier i every rank writes i into its cell, after it every rank reads all

@@ -112,6 +112,13 @@ def test_two_shot_one_launch_per_rank(world, tmp_path):
                     assert torch.equal(got, want), f"{tag} round {round_} rank {r} {what}"
 
 
+def test_reference_barrier_test(tmp_path):
+    """triton_barrier.py:155-190 as a per-rank program: 8 ranks, 32 blocks each, one launch per
+    rank; afterwards every rank's signal pad is all zero."""
+    codes, outs = run_ranks(8, tmp_path, "barrier_test")
+    assert codes == [0] * 8, "\n".join(outs)
+
+
 @pytest.mark.parametrize("world", [3, 8])
 def test_barriers_back_to_back_with_ranks_out_of_step(world, tmp_path):
     """A rank may enter its next barrier while a peer has seen, but not yet lowered, the flag of the
