@@ -57,6 +57,29 @@ def main():
         world.close()
         return 42 if reported else (0 if rank != 0 else 1)
 
+    if mode == "reference_mains":
+        # the self-tests at the bottom of the reference's four kernel files, with a process per rank
+        # as there: triton_one_shot_all_reduce_no_128.py:116-127, triton_reduce_scatter.py:185-211,
+        # triton_all_gather.py:117-133, triton_double_tree_allreduce.py:388-410
+        total = world_size * (world_size - 1) // 2
+        tensor = world.empty(8192, torch.bfloat16).fill_(rank)
+        world.barrier()
+        output = tccl_amd.one_shot_all_reduce(tensor)
+        assert output.eq(total).all().item(), "all-reduce"
+        share = tccl_amd.reduce_scatter(tensor)
+        assert share.shape == (8192 // world_size,) and share.eq(total).all().item(), "reduce-scatter"
+        gathered = tccl_amd.all_gather(tensor, world_size)
+        want = torch.arange(world_size, dtype=torch.bfloat16, device=tensor.device).unsqueeze(1).expand(world_size, 8192)
+        assert gathered.shape == (world_size, 8192) and gathered.eq(want).all().item(), "all-gather"
+        world.barrier()
+        if world_size in (2, 4, 8):
+            output = world.double_tree_all_reduce(tensor)
+            assert output.eq(total).all().item() and tensor.eq(total).all().item(), "double tree"
+        world.check()
+        print(f"rank {rank}: OUTPUT {world_size} {output[:4].tolist()}", flush=True)
+        world.close()
+        return 0
+
     if mode == "barrier_test":
         # the reference's own barrier test (triton_barrier.py:155-190): 32 blocks per rank, one
         # launch per rank, then look at the pad -- which must be all zero again

@@ -112,6 +112,15 @@ def test_two_shot_one_launch_per_rank(world, tmp_path):
                     assert torch.equal(got, want), f"{tag} round {round_} rank {r} {what}"
 
 
+@pytest.mark.parametrize("world", [8, 4])
+def test_reference_self_tests_with_a_process_per_rank(world, tmp_path):
+    """The `__main__` self-tests of the reference's kernel files (every rank fills its buffer
+    with its rank, the sum must be W(W-1)/2 everywhere), run the way the reference runs them:
+    one process per rank."""
+    codes, outs = run_ranks(world, tmp_path, "reference_mains")
+    assert codes == [0] * world, "\n".join(outs)
+
+
 def test_reference_barrier_test(tmp_path):
     """triton_barrier.py:155-190 as a per-rank program: 8 ranks, 32 blocks each, one launch per
     rank; afterwards every rank's signal pad is all zero."""
