@@ -402,6 +402,9 @@ def cold_ceilings(torch, lib, plib, device):
     out["write_64MiB_128KiB_tiles_gbs"] = round(W / (ms * 1e-3) / 1e9, 1)
     _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_write_small(base + k * W, W, s), 64), 128, 64)
     out["write_64MiB_32KiB_tiles_gbs"] = round(W / (ms * 1e-3) / 1e9, 1)
+    D = 256 << 20
+    _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_write_dense(base + k * D, D, s), 16), 48, 16)
+    out["write_256MiB_one_dense_window_gbs"] = round(D / (ms * 1e-3) / 1e9, 1)
     C = 128 << 20
     _, ms = time_steps(torch, lib, Rotation(lambda k: plib.tccl_probe_copy(base + (2 * k) * C, base + (2 * k + 1) * C, C, s), 16), 32, 16)
     out["copy_128MiB_gbs"] = round(2 * C / (ms * 1e-3) / 1e9, 1)

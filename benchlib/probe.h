@@ -19,8 +19,10 @@ extern "C" {
 int tccl_probe_read(const void *const *bufs, int world, size_t bytes_per_buffer, void *sink, void *stream);
 /* The write half: fills `bytes` at dst with a pattern, 32 stores per lane back to back. */
 int tccl_probe_write(void *dst, size_t bytes, void *stream);
-/* The same fill in 32 KiB tiles: the fastest way found to write HBM. */
+/* The same fill in 32 KiB tiles: the fastest way found to write HBM in tiles. */
 int tccl_probe_write_small(void *dst, size_t bytes, void *stream);
+/* pure write, one workgroup per compute unit, 4 KiB per workgroup per step: one dense window */
+int tccl_probe_write_dense(void *dst, size_t bytes, void *stream);
 /* One contiguous range read front to back by the whole GPU (grid-stride, streaming loads): the
  * fastest way found to read HBM, the reference point for every read rate in the benchmark. */
 int tccl_probe_read_dense(const void *buf, size_t bytes, void *sink, void *stream);

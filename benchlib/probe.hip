@@ -90,7 +90,7 @@ __global__ void __launch_bounds__(kPhasedBlock) probe_write_kernel(char *dst, si
 }
 
 // The same stores in 32 KiB tiles (8 per lane): four times as many workgroups, whose write fronts
-// move through memory as one dense window; the fastest way found to write HBM.
+// move through memory more closely together; the fastest way found to write HBM in tiles.
 __global__ void __launch_bounds__(kPhasedBlock) probe_write_small_kernel(char *dst, size_t bytes, uint32_t value)
 {
     constexpr int VECS = 8;
@@ -104,6 +104,21 @@ __global__ void __launch_bounds__(kPhasedBlock) probe_write_small_kernel(char *d
 #pragma unroll
     for (int k = 0; k < VECS; ++k)
         __builtin_amdgcn_raw_buffer_store_b128(v, rd, k * (kPhasedBlock * kVecBytes) + lane_off, 0, kAuxStoreStream);
+}
+
+// One workgroup per compute unit, each writing 4 KiB per step at a stride of the whole grid: the
+// GPU writes one dense 1 MiB window at a time with one wave per SIMD.  The fastest way found to
+// write HBM (more workgroups, or more bytes per workgroup per step, are slower); no kernel that
+// reads what it writes in tiles can write like this.
+__global__ void __launch_bounds__(kPhasedBlock) probe_write_dense_kernel(char *dst, size_t bytes, uint32_t value)
+{
+    constexpr size_t piece = static_cast<size_t>(kPhasedBlock) * kVecBytes;
+    const u32x4 v = {value, value + threadIdx.x, value ^ blockIdx.x, value};
+    for (size_t off = blockIdx.x * piece; off < bytes; off += gridDim.x * piece) {
+        const size_t left = bytes - off;
+        const __amdgpu_buffer_rsrc_t rd = tile_rsrc(dst + off, static_cast<uint32_t>(left < piece ? left : piece));
+        __builtin_amdgcn_raw_buffer_store_b128(v, rd, threadIdx.x * kVecBytes, 0, kAuxStoreStream);
+    }
 }
 
 template <int NSRC>
@@ -290,6 +305,16 @@ extern "C" int tccl_probe_write_small(void *dst, size_t bytes, void *stream)
     const size_t grid = (bytes + tile_bytes - 1) / tile_bytes;
     if (grid > 0x7FFFFFFFu) return TCCL_EINVAL;
     hipLaunchKernelGGL(probe_write_small_kernel, dim3(static_cast<unsigned>(grid)), dim3(kPhasedBlock), 0,
+                       static_cast<hipStream_t>(stream), static_cast<char *>(dst), bytes, 0x3F803F80u);
+    return hip_code(hipGetLastError());
+}
+
+extern "C" int tccl_probe_write_dense(void *dst, size_t bytes, void *stream)
+{
+    if (dst == nullptr) return TCCL_EINVAL;
+    if (bytes % kVecBytes != 0 || !aligned16(dst)) return TCCL_EALIGN;
+    if (bytes == 0) return TCCL_OK;
+    hipLaunchKernelGGL(probe_write_dense_kernel, dim3(probe_compute_units()), dim3(kPhasedBlock), 0,
                        static_cast<hipStream_t>(stream), static_cast<char *>(dst), bytes, 0x3F803F80u);
     return hip_code(hipGetLastError());
 }

@@ -14,6 +14,7 @@ SIGNATURES = {
     "tccl_probe_read": (_I, [_PP, _I, _SZ, _P, _P]),
     "tccl_probe_write": (_I, [_P, _SZ, _P]),
     "tccl_probe_write_small": (_I, [_P, _SZ, _P]),
+    "tccl_probe_write_dense": (_I, [_P, _SZ, _P]),
     "tccl_probe_read_dense": (_I, [_P, _SZ, _P, _P]),
     "tccl_probe_copy": (_I, [_P, _P, _SZ, _P]),
     "tccl_probe_sum_timed": (_I, [_PP, _P, _SZ, _P, _P]),

@@ -834,11 +834,13 @@ def test_probe_kernels_touch_what_they_say(_gpu_hygiene):
     for nbytes in [16, 128 * 1024 - 16, 128 * 1024 * 513 + 32, 64 << 20]:
         guard = 256
         region = torch.full((nbytes + 2 * guard,), 0xAB, dtype=torch.uint8, device=DEV)
-        assert lib.tccl_probe_write(region.data_ptr() + guard, nbytes, stream()) == 0
-        torch.cuda.synchronize()
-        assert bool((region[:guard] == 0xAB).all()) and bool((region[guard + nbytes:] == 0xAB).all())
-        words = region[guard:guard + nbytes].view(torch.int32)
-        assert bool((words[0::4] == 0x3F803F80).all()) and bool((words[3::4] == 0x3F803F80).all())
+        for write in (lib.tccl_probe_write, lib.tccl_probe_write_small, lib.tccl_probe_write_dense):
+            region.fill_(0xAB)
+            assert write(region.data_ptr() + guard, nbytes, stream()) == 0
+            torch.cuda.synchronize()
+            assert bool((region[:guard] == 0xAB).all()) and bool((region[guard + nbytes:] == 0xAB).all())
+            words = region[guard:guard + nbytes].view(torch.int32)
+            assert bool((words[0::4] == 0x3F803F80).all()) and bool((words[3::4] == 0x3F803F80).all())
     assert lib.tccl_probe_empty(stream()) == 0
     where = torch.full((2 * 512,), -1, dtype=torch.int32, device=DEV)
     assert lib.tccl_probe_placement(where.data_ptr(), 512, 100, stream()) == 0
