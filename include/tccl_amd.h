@@ -18,7 +18,10 @@
  *     wait/send flags (triton_double_tree_allreduce.py:175-225).  Two entry points keep the
  *     device-side protocol instead, between the virtual ranks' workgroups of one launch:
  *     tccl_double_tree_all_reduce_pipelined() and tccl_two_shot_all_reduce(); they take
- *     signal pads.
+ *     signal pads.  Where every rank is a process of its own on the same GPU (buffers and pads
+ *     exchanged with tccl_ipc_export/open), the same protocol runs between one launch per rank,
+ *     as in the reference: tccl_blockwise_barrier(), tccl_double_tree_all_reduce_pipelined_rank(),
+ *     tccl_two_shot_all_reduce_rank().
  *   - float sums: each bf16 is widened to fp32, accumulated from +0.0f in the order the
  *     sources are given, and rounded once (round-to-nearest-even) on store.  NaN sign
  *     and payload are not specified.
