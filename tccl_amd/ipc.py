@@ -70,6 +70,19 @@ class IpcWorld:
         self._pad_ptrs = self._exchange(self._alloc(self.PAD_BYTES), "pad")
         self._pad_array = _lib.ptr_array(self._pad_ptrs)
 
+    @classmethod
+    def from_env(cls, device="cuda:0", timeout_s: float = 60.0) -> "IpcWorld":
+        """The world a launcher describes in the environment, as the reference's programs read it
+        (triton_one_shot_all_reduce_no_128.py:106-108): RANK and WORLD_SIZE, plus
+        TCCL_RENDEZVOUS_DIR, the directory the ranks exchange their handles through
+        (``python -m tccl_amd.launch`` sets all three)."""
+        try:
+            rank, world_size = int(os.environ["RANK"]), int(os.environ["WORLD_SIZE"])
+            directory = os.environ["TCCL_RENDEZVOUS_DIR"]
+        except KeyError as e:
+            raise RuntimeError(f"{e.args[0]} is not set: start the program with python -m tccl_amd.launch") from None
+        return cls(rank, world_size, directory, device=device, timeout_s=timeout_s)
+
     # ---- plumbing
     def _alloc(self, nbytes: int) -> int:
         p = ctypes.c_void_p()

@@ -1,0 +1,54 @@
+"""Start a per-rank program once per rank on ONE GPU, the way the reference's programs are started
+by torchrun (triton_one_shot_all_reduce_no_128.py:99-110 reads RANK, LOCAL_RANK and WORLD_SIZE):
+
+    python -m tccl_amd.launch --nproc-per-node 8 program.py [arguments of the program ...]
+
+Every rank is a process of its own with RANK = 0 .. W-1, WORLD_SIZE = W, LOCAL_RANK = 0 (all ranks
+share the one GPU) and TCCL_RENDEZVOUS_DIR = a fresh directory through which the ranks exchange
+their buffer handles; ``tccl_amd.ipc.IpcWorld.from_env()`` in the program picks these up.  The
+launcher itself never touches the GPU.  Its exit code is the first non-zero exit code of a rank."""
+from __future__ import annotations
+
+import argparse
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="python -m tccl_amd.launch", description=__doc__.split("\n\n")[0])
+    ap.add_argument("--nproc-per-node", type=int, required=True, help="ranks (processes) to start, 1..8")
+    ap.add_argument("--timeout", type=float, default=600.0, help="seconds before ranks still running are stopped")
+    ap.add_argument("program", help="the per-rank program (a Python file)")
+    ap.add_argument("args", nargs=argparse.REMAINDER, help="its arguments")
+    ns = ap.parse_args(argv)
+    if not 1 <= ns.nproc_per_node <= 8:
+        ap.error("--nproc-per-node must be 1..8")
+    directory = tempfile.mkdtemp(prefix="tccl_rendezvous_")
+    procs = []
+    try:
+        for rank in range(ns.nproc_per_node):
+            env = dict(os.environ, RANK=str(rank), LOCAL_RANK="0", WORLD_SIZE=str(ns.nproc_per_node),
+                       TCCL_RENDEZVOUS_DIR=directory)
+            procs.append(subprocess.Popen([sys.executable, ns.program, *ns.args], env=env))
+        code = 0
+        for p in procs:
+            try:
+                rc = p.wait(timeout=ns.timeout)
+            except subprocess.TimeoutExpired:
+                rc = 124
+            if rc != 0 and code == 0:
+                code = rc
+        return code
+    finally:
+        for p in procs:                      # exactly the processes started here
+            if p.poll() is None:
+                p.kill()
+                p.wait()
+        shutil.rmtree(directory, ignore_errors=True)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

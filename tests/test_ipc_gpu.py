@@ -121,6 +121,17 @@ def test_reference_self_tests_with_a_process_per_rank(world, tmp_path):
     assert codes == [0] * world, "\n".join(outs)
 
 
+def test_launcher_runs_a_program_once_per_rank():
+    """python -m tccl_amd.launch: RANK / WORLD_SIZE / TCCL_RENDEZVOUS_DIR in the environment of
+    every rank, the exit code of a failing rank handed on."""
+    cmd = [sys.executable, "-m", "tccl_amd.launch", "--nproc-per-node", "8", os.path.join(ROOT, "tests", "ipc_env_program.py")]
+    done = subprocess.run(cmd, cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=150)
+    assert done.returncode == 0, done.stdout
+    assert done.stdout.count("OUTPUT") == 8 and "[28.0, 28.0, 28.0, 28.0]" in done.stdout
+    done = subprocess.run(cmd + ["7"], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=150)
+    assert done.returncode == 7, done.stdout
+
+
 def test_reference_barrier_test(tmp_path):
     """triton_barrier.py:155-190 as a per-rank program: 8 ranks, 32 blocks each, one launch per
     rank; afterwards every rank's signal pad is all zero."""
