@@ -1,5 +1,9 @@
 """Host-side logic that needs no GPU: the virtual-rank registry and the wrappers'
 preconditions (the reference's assertions, raised before anything is launched)."""
+import os
+import subprocess
+import sys
+
 import pytest
 import torch
 
@@ -77,3 +81,22 @@ def test_wrapper_preconditions_match_the_reference():
 def test_names():
     assert tccl_amd.reduce_scatter is tccl_amd.one_shot_reduce_scatter
     assert tccl_amd.all_gather is tccl_amd.one_shot_all_gather
+
+
+def test_launcher_sets_the_environment_and_hands_on_exit_codes(tmp_path):
+    """python -m tccl_amd.launch on a program that needs no GPU: every rank sees its RANK, the
+    common WORLD_SIZE and rendezvous directory; a failing rank's exit code is the launcher's."""
+    prog = tmp_path / "prog.py"
+    prog.write_text("import os, sys\n"
+                    "r, w, d = os.environ['RANK'], os.environ['WORLD_SIZE'], os.environ['TCCL_RENDEZVOUS_DIR']\n"
+                    "assert os.environ['LOCAL_RANK'] == '0' and os.path.isdir(d)\n"
+                    "open(os.path.join(sys.argv[1], 'seen' + r), 'w').write(w + ' ' + d)\n"
+                    "sys.exit(int(sys.argv[2]) if r == '2' else 0)\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, "-m", "tccl_amd.launch", "--nproc-per-node", "3", str(prog), str(tmp_path)]
+    assert subprocess.run(cmd + ["0"], cwd=root, timeout=60).returncode == 0
+    seen = [(tmp_path / f"seen{r}").read_text() for r in range(3)]
+    assert all(s.startswith("3 ") for s in seen) and len(set(seen)) == 1
+    assert not os.path.exists(seen[0].split(" ", 1)[1]), "the rendezvous directory is removed afterwards"
+    assert subprocess.run(cmd + ["5"], cwd=root, timeout=60).returncode == 5
+    assert subprocess.run(cmd[:4] + ["9", str(prog)], cwd=root, timeout=60, stderr=subprocess.DEVNULL).returncode == 2
