@@ -413,19 +413,57 @@ __global__ void __launch_bounds__(kPhasedBlock) tree_pipelined_kernel(PipeArgs a
 }
 
 // Workgroups per rank for `units` units of work (chunks, tiles) per rank, at most `most`.
-// Workgroup g takes units g, g + G, ...: what costs time is a last round that only part of
-// the grid takes part in, so the count that wastes the fewest workgroup-rounds wins (one that
-// divides `units` exactly wastes none: 128 for 1,024 chunks, 153 for 306 -- measured 5-12 %
-// better than their neighbours), among counts from 60 % of `most` upwards.  Ties go to a
-// multiple of 8 and then to the larger count: workgroups go to the 8 XCDs round-robin, so with
-// a multiple of 8 per rank, workgroup g of every rank shares an XCD and its L2, and part of
-// what a rank reads from a peer right after the peer wrote it never leaves the XCD (8 % of
-// the pipelined tree's reads and 29 % of the two-shot's, by the fetch counters).
-static size_t workgroups_per_rank(size_t units, size_t most)
+// Workgroup g takes units g, g + G, ...
+//
+// First choice: a count that gives every compute unit the same number of workgroups (G * world a
+// multiple of the units: 96, 128 or 160 per rank for a world of 8 on 256 units), at least three
+// per unit.  The hardware deals a grid out to the units evenly, so with any other count some
+// units carry one workgroup more than the rest and the launch lasts as long as they do: for the
+// two-shot all-reduce of 8 x 64 MiB, 128 per rank took 208 us, 120 took 222, 112 230, 104 241
+// and 103 (which wastes no workgroup-round on 513 tiles) 260.  Among the balanced counts the
+// one with the fewest unit-slots on the busiest compute unit wins -- per unit, workgroups x
+// full rounds, plus the partial last round -- then one that divides `units` exactly (128 for
+// 1,024 chunks), then the smaller or the larger as the kernel likes it (the two-shot kernel is
+// as fast with three workgroups per unit as with four and loses less in a partial last round:
+// 213 against 224 us for 513 tiles; the pipelined tree wants the most workgroups it can get: 96
+// per rank measured 10-15 % slower than 128 or 160).  Such counts are multiples of 8 per rank for worlds of 2, 4
+// and 8, so workgroup g of every rank shares an XCD and its L2 (workgroups go to the 8 XCDs
+// round-robin), and part of what a rank reads from a peer right after the peer wrote it never
+// leaves the XCD (8 % of the pipelined tree's reads and 29 % of the two-shot's, by the fetch
+// counters).
+// Where no balanced count fits (worlds of 5 and 7): the count from 60 % of `most` upwards that
+// wastes the fewest workgroup-rounds, ties to a multiple of 8 and then to the larger.
+static size_t workgroups_per_rank(size_t units, size_t most, int world, bool ties_to_larger)
 {
     if (most < 1) most = 1;
     if (units <= most) return units < 1 ? 1 : units;
-    size_t best = most, best_score = static_cast<size_t>(-1);
+    const size_t cus = static_cast<size_t>(compute_units());
+    const size_t w = static_cast<size_t>(world < 1 ? 1 : world);
+    size_t a = w, b = cus; // greatest common divisor
+    while (b != 0) {
+        const size_t t = a % b;
+        a = b;
+        b = t;
+    }
+    const size_t step = cus / (a > 0 ? a : 1);
+    size_t best = 0, best_cost = static_cast<size_t>(-1);
+    bool best_exact = false;
+    for (size_t g = step; step > 0 && g <= most; g += step) {
+        const size_t per_cu = g * w / cus;
+        if (per_cu < 3 && g + step <= most) continue; // too few waves to keep the memory system busy
+        const size_t full = units / g, rem = units % g;
+        const size_t last = (rem * w + cus - 1) / cus;
+        const size_t cost = per_cu * full + (last < per_cu ? last : per_cu);
+        const bool exact = rem == 0;
+        if (cost < best_cost || (cost == best_cost && (exact != best_exact ? exact : ties_to_larger))) {
+            best = g;
+            best_cost = cost;
+            best_exact = exact;
+        }
+    }
+    if (best != 0) return best;
+    best = most;
+    size_t best_score = static_cast<size_t>(-1);
     const size_t least = most * 6 / 10 > 0 ? most * 6 / 10 : 1;
     for (size_t g = most; g >= least; --g) {
         const size_t rounds = (units + g - 1) / g;
@@ -470,7 +508,7 @@ static int launch_pipelined(const PipeArgs &a, int wgs_wanted, int world, size_t
         if (per_rank < 1) per_rank = 1;
         if (static_cast<size_t>(per_rank) > slots) per_rank = static_cast<int>(slots);
     } else {
-        per_rank = static_cast<int>(workgroups_per_rank(slots, resident / world));
+        per_rank = static_cast<int>(workgroups_per_rank(slots, static_cast<size_t>(resident / world), world, true));
     }
     PipeArgs args = a;
     args.wgs_per_rank = per_rank;
@@ -826,7 +864,7 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, cons
         if (per_rank > fit) per_rank = fit;
     } else {
         const size_t most = static_cast<size_t>(resident / W);
-        per_rank = workgroups_per_rank(tiles, most < fit ? most : fit);
+        per_rank = workgroups_per_rank(tiles, most < fit ? most : fit, W, false);
     }
     a.wgs_per_rank = static_cast<int>(per_rank);
     SignallingLaunch guard(s); // from here on the stream is behind the device's previous signalling kernel
