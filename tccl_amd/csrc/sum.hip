@@ -80,10 +80,12 @@ static hipError_t launch_sum_nsrc(const char *const *srcs, int nsrc, char *out, 
 
 template <class Sum, int NSRC, int U, bool FULL>
 __global__ void __launch_bounds__(kPhasedBlock)
-sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_t tail_first, size_t numel)
+sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_t tile_bytes, size_t tail_first,
+                  size_t numel)
 {
+    // tile_bytes <= what kcount iterations cover; where it is less, the lanes beyond it load
+    // nothing and store nothing (the tile's buffer descriptor ends there)
     constexpr int KMAX = kPhasedVecs / U;
-    const size_t tile_bytes = static_cast<size_t>(kcount) * (kPhasedBlock * U * kVecBytes);
     const size_t off = blockIdx.x * tile_bytes;
     const size_t left = bytes > off ? bytes - off : 0;
     const uint32_t valid = static_cast<uint32_t>(left < tile_bytes ? left : tile_bytes);
@@ -155,15 +157,22 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
     constexpr size_t span = static_cast<size_t>(kPhasedBlock) * U; // vectors per iteration
     const size_t nvec = numel / per_vec;
     size_t wgs = (cfg && cfg->grid > 0) ? static_cast<size_t>(cfg->grid) : static_cast<size_t>(compute_units()) * 2;
-    size_t kcount;
+    size_t kcount, small_tile_vec = 0;
     if (cfg && cfg->tile_iters > 0) {
         kcount = static_cast<size_t>(cfg->tile_iters) > kmax ? kmax : cfg->tile_iters;
     } else if (small_input) {
-        // one launch of at most two workgroups per compute unit, with the fewest iterations that
-        // cover the input (see launch_phased)
-        kcount = (nvec + wgs * span - 1) / (wgs * span);
+        // one launch of one or two workgroups per compute unit (two where that leaves every
+        // workgroup at least a full iteration), the input cut into that many equal tiles whatever
+        // its size -- every compute unit carries the same load -- and the fewest iterations
+        // that cover a tile (see launch_phased)
+        if (nvec < wgs * span) wgs /= 2;
+        small_tile_vec = (nvec + wgs - 1) / wgs;
+        kcount = (small_tile_vec + span - 1) / span;
         if (kcount < 1) kcount = 1;
-        if (kcount > kmax) kcount = kmax;
+        if (kcount > kmax) { // cannot happen below kSmallInputBytes; keeps the plan valid if that grows
+            kcount = kmax;
+            small_tile_vec = kcount * span;
+        }
     } else if (NSRC <= 3 && !(cfg && cfg->grid > 0) &&
                nvec * kVecBytes >= (static_cast<size_t>(NSRC <= 2 ? 48 : 96) << 20)) {
         // With three sources or fewer a quarter or more of the traffic is writes and there
@@ -187,7 +196,7 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
         if (kcount > kmax) kcount = kmax;
     }
     if (wgs > (static_cast<size_t>(1) << 30)) wgs = static_cast<size_t>(1) << 30; // grid dimension limit
-    const size_t tile_vec = kcount * span;
+    const size_t tile_vec = small_tile_vec > 0 ? small_tile_vec : kcount * span;
     const size_t slice_vec = wgs * tile_vec;
     // full-size tiles of many sources, launch shape left to the library: unequal tiles for even and
     // odd XCDs (see sum_phased_skewed_kernel)
@@ -213,11 +222,11 @@ static hipError_t launch_phased_u(const char *const *srcs, char *out, size_t num
         } else if (kcount == kmax)
             hipLaunchKernelGGL((sum_phased_kernel<Sum, NSRC, U, true>), dim3(static_cast<unsigned>(grid)),
                                dim3(kPhasedBlock), 0, stream, t, out + off * kVecBytes, n * kVecBytes,
-                               static_cast<int>(kcount), rel_first, rel_numel);
+                               static_cast<int>(kcount), tile_vec * kVecBytes, rel_first, rel_numel);
         else
             hipLaunchKernelGGL((sum_phased_kernel<Sum, NSRC, U, false>), dim3(static_cast<unsigned>(grid)),
                                dim3(kPhasedBlock), 0, stream, t, out + off * kVecBytes, n * kVecBytes,
-                               static_cast<int>(kcount), rel_first, rel_numel);
+                               static_cast<int>(kcount), tile_vec * kVecBytes, rel_first, rel_numel);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         off += n;
@@ -238,7 +247,10 @@ static hipError_t launch_phased(const char *const *srcs, char *out, size_t numel
         // iteration), as long as that still gives every compute unit a workgroup.  Measured on
         // buffers rotated so that nothing is cached, against the plans for larger inputs: 8 sources
         // 2 MiB -18 %, 4 MiB -12 %, 8 MiB -5 %; 4 sources -16 %, -8 %, -6 %; 2 sources 8 MiB -6 %;
-        // at 16 MiB the difference is gone.
+        // at 16 MiB the difference is gone.  The input is cut into exactly as many equal tiles as
+        // there are workgroups (a tile need not be a whole number of iterations), so sizes between the
+        // powers of two do not leave half of the compute units with twice the work: 4.5 MiB 11.1 ->
+        // 9.4 us, 5 MiB 11.8 -> 10.1 us.
         constexpr size_t per_vec = kVecBytes / Sum::kElemBytes;
         const size_t nvec = numel / per_vec;
         const size_t one_per_cu = static_cast<size_t>(compute_units()) * kPhasedBlock;
