@@ -651,9 +651,7 @@ def main():
     wall_ms, dev_ms = time_steps(torch, lib, step, args.steps, args.warmup)
     gbs_wall = algo_bytes / (wall_ms * 1e-3) / 1e9
     gbs_dev = algo_bytes / (dev_ms * 1e-3) / 1e9
-    # allocated only now: the step's output is then the allocation right behind the eight inputs (with a
-    # 256 MiB buffer between them the launch measured 0.6 us slower: where buffers lie matters to HBM)
-    noise = Noise(torch, device)
+    noise = Noise(torch, device)         # filler for every later buffer; not needed before this point
 
     # The same step rotated over 8 disjoint sets of inputs AND outputs (4.6 GiB touched between
     # two uses of any byte).  On one set the 256 MB memory-side cache absorbs the 64 MiB of
