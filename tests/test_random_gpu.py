@@ -48,6 +48,40 @@ def _oracle(c_oracle, bufs):
     return torch.from_numpy(c_oracle.all_reduce_f32([b.numpy() for b in bufs]))
 
 
+def _default_plan_cases(n, seed):
+    """Sizes across every launch plan the library chooses by itself (no launch overrides): the
+    grid-stride kernel, the plan for small inputs, partial and full tiles, unequal interleaved
+    tiles, several launches per call, the single-launch rule for few sources."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        world = int(rng.integers(1, 9))
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+        esize = 2 if dtype == torch.bfloat16 else 4
+        mib = float(rng.choice([1.7, 2.0, 2.3, 3.1, 4.0, 4.6, 6.5, 8.0, 8.1, 13.0, 24.0, 31.9, 32.0, 47.0, 63.9, 64.0, 65.0, 100.0]))
+        numel = int(mib * (1 << 20)) // esize + int(rng.integers(-40, 41))
+        out.append((i, world, dtype, numel))
+    return out
+
+
+@pytest.mark.parametrize("case", _default_plan_cases(36, 77), ids=lambda c: f"plan{c[0]}")
+def test_random_sizes_default_plans(case, c_oracle):
+    i, world, dtype, numel = case
+    lib = tccl_amd.load_library()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = torch.Generator().manual_seed(5000 + i)
+    first = torch.randn(numel, generator=g).to(dtype) if dtype == torch.bfloat16 else torch.rand(numel, generator=g) * 2 - 1
+    bufs = [first.roll(r * 7919) for r in range(world)]
+    dev = [b.to(DEV) for b in bufs]
+    ptrs = _lib.ptr_array([d.data_ptr() for d in dev])
+    dt = _lib.TCCL_BF16 if dtype == torch.bfloat16 else _lib.TCCL_F32
+    out = torch.full((numel + 32,), 3.0, dtype=dtype, device=DEV)
+    print(f"plan case {i}: world={world} dtype={dtype} numel={numel}", flush=True)
+    assert lib.tccl_all_reduce_sum(ptrs, world, out.data_ptr(), numel, dt, stream) == 0
+    assert_bit_equal(out[:numel], _oracle(c_oracle, bufs), "all-reduce")
+    assert out[numel:].eq(3.0).all().item(), "wrote past the end"
+
+
 @pytest.mark.parametrize("case", _cases(80, 20240607), ids=lambda c: f"case{c[0]}")
 def test_random_all_reduce_and_reduce_scatter(case, c_oracle):
     i, world, dtype, numel, cfgd = case
