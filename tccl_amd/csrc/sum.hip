@@ -307,6 +307,9 @@ int sum_streams(const void *const *srcs, int nsrc, void *out, size_t numel, int 
     }
     if (!aligned16(out)) return TCCL_EALIGN;
     if (numel == 0) return TCCL_OK;
+    // a configuration that overrides nothing is no configuration: the library's own plans apply
+    if (cfg && cfg->block == 0 && cfg->unroll == 0 && cfg->grid == 0 && cfg->tile_iters == 0 && cfg->flags == 0)
+        cfg = nullptr;
 
     const size_t nvec = numel * static_cast<size_t>(esize) / kVecBytes;
     const char *const *s = reinterpret_cast<const char *const *>(srcs);
