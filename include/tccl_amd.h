@@ -313,7 +313,9 @@ int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void *const *sig
  * in a static device array inside the library (TCCL_STATIC_SCRATCH_BYTES per GPU, held from
  * the moment the library is loaded until the process ends), and the call allocates nothing on
  * the device or the host: it enqueues one small kernel that clears the pads and then the
- * all-reduce itself.  Limits: world <= TCCL_MAX_WORLD and at most TCCL_STATIC_MAX_WORKGROUPS
+ * all-reduce itself.  (Set-up, once per device: the first call looks up the array's device
+ * address, and the first signalling launch of the process outside graph capture creates the
+ * one HIP event with which the library chains such launches.)  Limits: world <= TCCL_MAX_WORLD and at most TCCL_STATIC_MAX_WORKGROUPS
  * workgroups per rank; a cfg->workgroups beyond world * TCCL_STATIC_MAX_WORKGROUPS is refused
  * with TCCL_ESCRATCH (numel itself is not limited: the pads hold one flag per workgroup and
  * peer, whatever the size).  Every call on a GPU uses that GPU's one array: calls that overlap
