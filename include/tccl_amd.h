@@ -64,7 +64,8 @@ typedef enum {
 } tccl_dtype_t;
 
 /* Launch shape override, for tuning and tests.  Any field left 0 is chosen by the
- * library (all fields 0 is the same as passing NULL: the library's own launch plans apply).  The reference hard-codes its shape in each wrapper
+ * library (all fields 0 is the same as passing NULL: the library's own launch plans
+ * apply).  The reference hard-codes its shape in each wrapper
  * (triton_one_shot_all_reduce_no_128.py:68-71: 24 blocks x 512 lanes). */
 typedef struct {
     int block;      /* threads per workgroup: 64, 128, 256 or 512 */
