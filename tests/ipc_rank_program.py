@@ -80,6 +80,42 @@ def main():
         world.close()
         return 0
 
+    if mode == "graph":
+        # [barrier, all-reduce, barrier] recorded once into a HIP graph by every rank and replayed with
+        # new inputs: the barrier needs no host-side state (its pads reset themselves), which is what
+        # the reference means by graph-friendly (triton_barrier.py:47-54)
+        numel = 8 * 3001
+        tensor = world.empty(numel, torch.bfloat16)
+        out = torch.empty(numel, dtype=torch.bfloat16, device=tensor.device)
+
+        def enqueue():
+            world.barrier()
+            tccl_amd.one_shot_all_reduce(tensor, out=out)
+            world.barrier()
+
+        tensor.fill_(rank)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            enqueue()                                  # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        world.host_barrier()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            enqueue()
+        for rep in range(4):
+            torch.manual_seed(100 * rep + rank)
+            tensor.copy_(torch.randn(numel, dtype=torch.bfloat16))
+            out.zero_()
+            graph.replay()
+            world.check()
+            save(directory, f"graph.{rep}", rank, out)
+            world.host_barrier()                       # nobody refills before everybody has saved
+        print(f"rank {rank}: graph replayed 4 times", flush=True)
+        world.close()
+        return 0
+
     if mode == "barrier_test":
         # the reference's own barrier test (triton_barrier.py:155-190): 32 blocks per rank, one
         # launch per rank, then look at the pad -- which must be all zero again

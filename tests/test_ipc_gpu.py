@@ -132,6 +132,19 @@ def test_launcher_runs_a_program_once_per_rank():
     assert done.returncode == 7, done.stdout
 
 
+def test_barrier_and_collective_replayed_from_a_graph_in_every_process(tmp_path):
+    """The barrier is graph-friendly in the reference's sense (triton_barrier.py:47-54): every rank
+    records [barrier, all-reduce, barrier] into a HIP graph once and replays it four times with new
+    inputs; each replay against the oracle."""
+    world, numel = 8, 8 * 3001
+    codes, outs = run_ranks(world, tmp_path, "graph")
+    assert codes == [0] * world, "\n".join(outs)
+    for rep in range(4):
+        want = torch_ref.all_reduce(seeded_randn(world, numel, seed_base=100 * rep)).view(torch.int16)
+        for r in range(world):
+            assert torch.equal(load(tmp_path, f"graph.{rep}", r, torch.bfloat16).view(torch.int16), want), f"replay {rep} rank {r}"
+
+
 def test_reference_barrier_test(tmp_path):
     """triton_barrier.py:155-190 as a per-rank program: 8 ranks, 32 blocks each, one launch per
     rank; afterwards every rank's signal pad is all zero."""
