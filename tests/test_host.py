@@ -100,3 +100,11 @@ def test_launcher_sets_the_environment_and_hands_on_exit_codes(tmp_path):
     assert not os.path.exists(seen[0].split(" ", 1)[1]), "the rendezvous directory is removed afterwards"
     assert subprocess.run(cmd + ["5"], cwd=root, timeout=60).returncode == 5
     assert subprocess.run(cmd[:4] + ["9", str(prog)], cwd=root, timeout=60, stderr=subprocess.DEVNULL).returncode == 2
+
+
+def test_world_from_environment_needs_a_launcher(monkeypatch):
+    from tccl_amd import ipc
+    for name in ("RANK", "WORLD_SIZE", "TCCL_RENDEZVOUS_DIR"):
+        monkeypatch.delenv(name, raising=False)
+    with pytest.raises(RuntimeError, match="tccl_amd.launch"):
+        ipc.IpcWorld.from_env()
