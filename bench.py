@@ -46,7 +46,11 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "headline_traffic.json")
 ONLY_OPS = ["all_reduce", "all_reduce_rotated", "probe_read", "probe_write", "reduce_scatter_bf16", "reduce_scatter_f32",
             "all_gather_bf16", "all_gather_f32", "all_gather_int8", "tree_reduce_c0", "tree_reduce_c1",
             "tree_reduce_c2", "tree_copy_1", "tree_copy_2", "double_tree_level", "double_tree_pipelined",
-            "double_tree_pipelined_drawn", "two_shot", "two_shot_drawn", "copy_calibration", "placement", "ceilings", "phase_timing"]
+            "double_tree_pipelined_drawn", "two_shot", "two_shot_drawn", "copy_calibration", "placement", "ceilings", "phase_timing", "floor"]
+# the all-reduce at the sizes of the sweep, rotated cold as the sweep does: c1 = the CPU-runnable shape (W=8 x 8 MiB)
+SWEEP_OPS = {"c1": (8, 8)}
+SWEEP_OPS.update({f"all_reduce_w{w}_{m}MiB": (w, m) for w in (2, 4, 8) for m in (4, 16, 64, 256)})
+ONLY_OPS += list(SWEEP_OPS)
 
 
 def parse_args():
@@ -68,6 +72,10 @@ def parse_args():
                         "run of this command holds a kernel of known traffic to scale the counters by")
     p.add_argument("--only", choices=ONLY_OPS,
                    help="run this one operation alone (--steps launches after --warmup) and print a small JSON line")
+    p.add_argument("--stamps", action="store_true",
+                   help="with --only OP: run OP through benchlib/libtccl_amd_stamped.so (the library's own kernels with "
+                        "wall-clock stamps per workgroup) and print when the workgroups start, get their first data, finish "
+                        "reading and finish writing, per XCD")
     return p.parse_args()
 
 
@@ -258,6 +266,25 @@ class Ops:
         fn = Rotation(lambda k: self.tccl_amd.one_shot_all_reduce(gs[k].tensor(0), out=outs[k]), nsets)
         return fn, nbytes, "sum_phased_skewed_kernel<Bf16Sum, 8>"
 
+    def all_reduce_cold(self, world, mib):
+        """The sweep's protocol: W buffers of `mib` MiB bf16 through the C entry point, rotated over
+        enough buffer sets that COLD_BYTES lie between two uses of a byte."""
+        torch, nbytes = self.torch, mib << 20
+        numel = nbytes // 2
+        touched = (world + 1) * nbytes
+        nsets = sets_for(touched)
+        sets = []
+        for k in range(nsets):
+            bufs = [self.noise.fill(torch.empty(numel, dtype=torch.bfloat16, device=self.device), 13 * k + r)
+                    for r in range(world)]
+            o = torch.empty(numel, dtype=torch.bfloat16, device=self.device)
+            sets.append((bufs, o, ctypes.cast((ctypes.c_void_p * world)(*[b.data_ptr() for b in bufs]),
+                                               ctypes.POINTER(ctypes.c_void_p))))
+        self.keep.append(sets)
+        stream = raw_stream(torch)
+        fn = Rotation(lambda k: self.lib.tccl_all_reduce_sum(sets[k][2], world, sets[k][1].data_ptr(), numel, 0, stream), nsets)
+        return fn, touched, "sum_phased*_kernel<Bf16Sum, %d, ...>" % world
+
     def probe_read(self):
         torch = self.torch
         gs = self._worlds(1, WORLD, BYTES_PER_BUF // 2, torch.bfloat16)
@@ -357,6 +384,8 @@ class Ops:
 
     def get(self, name):
         torch = self.torch
+        if name in SWEEP_OPS:
+            return self.all_reduce_cold(*SWEEP_OPS[name])
         if name == "all_reduce":
             return self.all_reduce(False)
         if name == "all_reduce_rotated":
@@ -444,7 +473,103 @@ def phase_timing(torch, tccl_amd, plib, device, launches=48):
         tccl_amd.unregister(g)
 
 
+class _DeviceWords:
+    """Device memory that torch does not own, seen through ``__cuda_array_interface__``."""
+
+    def __init__(self, ptr, nbytes):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 2}
+
+
+def stamp_table(args, torch, tccl_amd, lib, device, burst=8):
+    """--only OP --stamps: OP through the stamped build of the library (every kernel of the library records
+    the 100 MHz wall clock per workgroup: start, first iteration's data there, last load reduced, last store
+    acknowledged).  Launches go out in bursts of `burst` back to back (rotating over the operation's buffer
+    sets as always); the stamps of a burst's last launch are read after it, `--steps` bursts in all."""
+    ptr, slots, room = ctypes.c_void_p(), ctypes.c_int(), ctypes.c_int()
+    assert lib.tccl_stamp_buffer(ctypes.byref(ptr), ctypes.byref(slots), ctypes.byref(room)) == 0
+    words = torch.as_tensor(_DeviceWords(ptr.value, 8 * slots.value * room.value), device=device).view(torch.int64)
+    words = words.view(room.value, slots.value)
+    noise = Noise(torch, device)
+    ops = Ops(torch, tccl_amd, lib, None, noise, device)
+    fn, nbytes, kernel = ops.get(args.only)
+    stream = raw_stream(torch)
+    ev = HipEvents(lib, 2)
+    for _ in range(max(args.warmup, burst)):
+        fn()
+    tables, event_us = [], []
+    for _ in range(args.steps):
+        words.zero_()
+        torch.cuda.synchronize()
+        ev.record(0, stream)
+        for _ in range(burst):
+            fn()
+        ev.record(1, stream)
+        torch.cuda.synchronize()
+        event_us.append(ev.elapsed_ms(0, 1) * 1e3 / burst)
+        w = words.cpu()
+        tables.append(w[w[:, 0] != 0].double())
+    ev.close()
+    n = min(t.shape[0] for t in tables)
+    assert all(t.shape[0] == n for t in tables), "the operation's launches differ in their grids"
+    t = torch.stack(tables)                                              # [bursts, workgroups, 4]
+    t = (t - t[:, :, 0].min(dim=1, keepdim=True)[0].unsqueeze(-1)) * 0.01      # us after the launch's first start
+    for slot in (1, 2):                                                  # kernels without those marks leave zeros
+        if float(tables[0][:, slot].max()) == 0.0:
+            t[:, :, slot] = float("nan")
+    span = t[:, :, 3].max(dim=1)[0]
+    b = torch.arange(n)
+    cus = 256
+    rounds = max(1, -(-n // cus))
+    print(f"Operation: bench.py --only {args.only} --stamps --steps {args.steps} --warmup {args.warmup}   kernel: {kernel}")
+    print(f"{n} workgroups stamped in the last launch of each burst of {burst} back-to-back calls, mean over {args.steps} bursts; "
+          f"algorithmic bytes per call {nbytes:,}")
+    print(f"HIP events over a burst: {statistics.mean(event_us):.2f} us per call (min {min(event_us):.2f}, max {max(event_us):.2f})")
+    print(f"first workgroup's start to last store acknowledged: mean {float(span.mean()):.2f} us, min {float(span.min()):.2f}, "
+          f"max {float(span.max()):.2f}   -> {nbytes / float(span.mean()) / 1e3:.0f} GB/s inside the launch")
+    if rounds > 1 and float(t[:, b // cus == 1, 0].mean()) > 0.2 * float(span.mean()):
+        print("NOTE: the second workgroup of a compute unit started only when the first had finished: the stamped build of this kernel "
+              "needs more registers than the product's and does not fit two per unit, so this table does not show the product's launch")
+    print("times in us after the launch's first workgroup started; 'k-th on its unit' = workgroup index // 256")
+    print("XCD  k-th on its unit   start mean  start max | first data mean   max | last load reduced mean    max | last store acked mean    max")
+    for x in range(8):
+        for k in range(rounds):
+            sel = (b % 8 == x) & (b // cus == k)
+            if int(sel.sum()) == 0:
+                continue
+            c = [t[:, sel, i] for i in range(4)]
+            f = lambda v: float(v.mean())
+            m = lambda v: float(v.max(dim=1)[0].mean())
+            print(f"{x:3d}  {k:3d}              {f(c[0]):10.2f}  {m(c[0]):9.2f} | {f(c[1]):15.2f} {m(c[1]):7.2f} | "
+                  f"{f(c[2]):22.2f} {m(c[2]):7.2f} | {f(c[3]):21.2f} {m(c[3]):7.2f}")
+    allf = lambda i: float(t[:, :, i].mean())
+    allm = lambda i: float(t[:, :, i].max(dim=1)[0].mean())
+    print(f"all                   {allf(0):10.2f}  {allm(0):9.2f} | {allf(1):15.2f} {allm(1):7.2f} | "
+          f"{allf(2):22.2f} {allm(2):7.2f} | {allf(3):21.2f} {allm(3):7.2f}")
+    ops.close()
+
+
+def floor(args, torch, lib, plib, device):
+    """What a short streaming kernel costs whatever it moves: an empty grid of 512 x 256 lanes, and the
+    same grid with every lane loading one vector and storing it (data that is in no cache)."""
+    arena = torch.empty(2 << 30, dtype=torch.uint8, device=device)
+    arena.view(torch.int32).fill_(0x3C003C00)
+    s = raw_stream(torch)
+    base, half, step = arena.data_ptr(), 1 << 30, 4 << 20
+    line = {"only": "floor", "steps": args.steps, "warmup": args.warmup}
+    for wgs in (256, 512):
+        _, ms = time_steps(torch, lib, lambda: plib.tccl_probe_empty_grid(wgs, s), args.steps, args.warmup)
+        line[f"empty_grid_{wgs}_us"] = round(ms * 1e3, 2)
+        fn = Rotation(lambda k: plib.tccl_probe_touch(base + k * step, base + half + k * step, wgs, s), half // step)
+        _, ms = time_steps(torch, lib, fn, args.steps, args.warmup)
+        line[f"touch_{wgs}_us"] = round(ms * 1e3, 2)
+    print(json.dumps(line), flush=True)
+
+
 def run_only(args, torch, tccl_amd, lib, plib, device):
+    if args.only == "floor":
+        return floor(args, torch, lib, plib, device)
+    if args.stamps:
+        return stamp_table(args, torch, tccl_amd, lib, device)
     if args.only == "placement":
         return placement(torch, plib, device)
     if args.only == "phase_timing":
@@ -626,6 +751,14 @@ def main():
     import torch
     import tccl_amd
     from benchlib import probe
+    if args.stamps:
+        # measurement build of the same sources (benchlib/stamped.hip); never the product's library
+        if not args.only:
+            sys.exit("--stamps needs --only OP")
+        from tccl_amd import _lib
+        _lib.LIB_PATH = os.path.join(ROOT, "benchlib", "libtccl_amd_stamped.so")
+        _lib.SIGNATURES["tccl_stamp_buffer"] = (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int),
+                                                               ctypes.POINTER(ctypes.c_int)])
     lib = tccl_amd.load_library()
     plib = probe.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"

@@ -35,6 +35,11 @@ int tccl_probe_copy(const void *src, void *dst, size_t bytes, void *stream);
 int tccl_probe_sum_timed(const void *const *bufs, void *out, size_t bytes_per_buffer, long long *stamps, void *stream);
 /* One empty kernel: what a timed single launch costs when the kernel does nothing. */
 int tccl_probe_empty(void *stream);
+/* An empty kernel of `workgroups` x 256 lanes, and the same grid with every lane loading one
+ * 16-byte vector from src and storing it to dst (both workgroups x 4 KiB): what a short
+ * streaming kernel costs whatever it moves. */
+int tccl_probe_empty_grid(int workgroups, void *stream);
+int tccl_probe_touch(const void *src, void *dst, int workgroups, void *stream);
 /* out[2*b] = HW_REG_HW_ID, out[2*b+1] = HW_REG_XCC_ID of workgroup b of a grid of `workgroups`
  * x 256 lanes, each holding its slot for hold_us microseconds. */
 int tccl_probe_placement(uint32_t *out, int workgroups, int hold_us, void *stream);

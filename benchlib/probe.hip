@@ -280,6 +280,21 @@ __global__ void __launch_bounds__(kPhasedBlock) probe_sum_timed_kernel(ProbeSrc<
 
 __global__ void probe_empty_kernel() {}
 
+// The same grid as a sum launch doing nothing, and doing the least a streaming kernel can do:
+// every lane loads one vector and stores it (one round trip to memory each way).  Their
+// durations are the part of a short kernel's time that does not depend on its bytes.
+__global__ void __launch_bounds__(kPhasedBlock) probe_empty_grid_kernel() {}
+
+__global__ void __launch_bounds__(kPhasedBlock) probe_touch_kernel(const char *src, char *dst)
+{
+    const uint32_t bytes = kPhasedBlock * kVecBytes;
+    const size_t off = static_cast<size_t>(blockIdx.x) * bytes;
+    const __amdgpu_buffer_rsrc_t rs = tile_rsrc(src + off, bytes);
+    const __amdgpu_buffer_rsrc_t rd = tile_rsrc(dst + off, bytes);
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, threadIdx.x * kVecBytes, 0, kAuxLoadStream);
+    __builtin_amdgcn_raw_buffer_store_b128(v, rd, threadIdx.x * kVecBytes, 0, kAuxStoreStream);
+}
+
 // Every workgroup holds its slot for `hold_ticks` of the 100 MHz wall clock (so that the whole
 // grid is resident together) and reports the XCD and the hardware id it ran on.
 __global__ void __launch_bounds__(kPhasedBlock) probe_placement_kernel(uint32_t *out, long long hold_ticks)
@@ -360,6 +375,21 @@ extern "C" int tccl_probe_sum_timed(const void *const *bufs, void *out, size_t b
 extern "C" int tccl_probe_empty(void *stream)
 {
     hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream));
+    return hip_code(hipGetLastError());
+}
+
+extern "C" int tccl_probe_empty_grid(int workgroups, void *stream)
+{
+    if (workgroups < 1 || workgroups > 65536) return TCCL_EINVAL;
+    hipLaunchKernelGGL(probe_empty_grid_kernel, dim3(workgroups), dim3(kPhasedBlock), 0, static_cast<hipStream_t>(stream));
+    return hip_code(hipGetLastError());
+}
+
+extern "C" int tccl_probe_touch(const void *src, void *dst, int workgroups, void *stream)
+{
+    if (src == nullptr || dst == nullptr || workgroups < 1 || workgroups > 65536) return TCCL_EINVAL;
+    hipLaunchKernelGGL(probe_touch_kernel, dim3(workgroups), dim3(kPhasedBlock), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const char *>(src), static_cast<char *>(dst));
     return hip_code(hipGetLastError());
 }
 

@@ -78,6 +78,23 @@ def build_probe(verbose: bool = False) -> str:
     return out
 
 
+def build_stamped(verbose: bool = False) -> str:
+    """Compile the measurement build of the library (benchlib/stamped.hip: every csrc/*.hip as one
+    translation unit with TCCL_STAMPS defined) into benchlib/libtccl_amd_stamped.so.  Loaded by
+    ``bench.py --only OP --stamps`` only; no part of the product."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "benchlib", "stamped.hip")
+    out = os.path.join(root, "benchlib", "libtccl_amd_stamped.so")
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", src, "-o", out + ".tmp"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on stamped.hip:\n{proc.stdout}\n{proc.stderr}")
+    os.replace(out + ".tmp", out)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 def build_c_client(verbose: bool = False) -> str:
     """Compile the plain C client of the library (tests/c_client) next to its source."""
     root = os.path.dirname(HERE)
@@ -99,5 +116,6 @@ def build_c_client(verbose: bool = False) -> str:
 if __name__ == "__main__":
     build(verbose=True)
     build_probe(verbose=True)
+    build_stamped(verbose=True)
     build_c_client(verbose=True)
     sys.exit(0)

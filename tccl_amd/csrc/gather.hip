@@ -17,13 +17,16 @@ template <int UNROLL, bool NTL, bool NTS>
 __global__ void __launch_bounds__(kMaxBlock)
 pack_kernel(RowTable rows, int world, char *out, size_t row_vecs, int tile_iters, int xcd_contiguous)
 {
+    TCCL_STAMP(0, false);
     pack_rows<UNROLL, NTL, NTS>(rows.p, world, out, row_vecs, tile_iters, xcd_contiguous != 0);
+    TCCL_STAMP(3, true);
 }
 
 template <int NDST, int UNROLL, bool NTL, bool NTS>
 __global__ void __launch_bounds__(kMaxBlock)
 copy_kernel(const char *src, char *dst0, char *dst1, size_t nvec, int tile_iters, int xcd_contiguous)
 {
+    TCCL_STAMP(0, false);
     if constexpr (NDST == 2) {
         char *const dst[2] = {dst0, dst1};
         copy_range<2, UNROLL, NTL, NTS>(src, dst, nvec, tile_iters, xcd_contiguous != 0);
@@ -31,6 +34,7 @@ copy_kernel(const char *src, char *dst0, char *dst1, size_t nvec, int tile_iters
         char *const dst[1] = {dst0};
         copy_range<1, UNROLL, NTL, NTS>(src, dst, nvec, tile_iters, xcd_contiguous != 0);
     }
+    TCCL_STAMP(3, true);
 }
 
 template <int UNROLL, bool NTL, bool NTS>

@@ -17,8 +17,10 @@ template <class Sum, int NSRC, int UNROLL, bool NTL, bool NTS>
 __global__ void __launch_bounds__(kMaxBlock)
 sum_kernel(SrcTable<NSRC> src, char *out, size_t numel, int tile_iters, int xcd_contiguous)
 {
+    TCCL_STAMP(0, false);
     char *const dst[1] = {out};
     sum_range<Sum, NSRC, 1, UNROLL, NTL, NTS>(src.p, dst, numel, tile_iters, xcd_contiguous != 0);
+    TCCL_STAMP(3, true);
 }
 
 template <class Sum, int NSRC, int UNROLL, bool NTL, bool NTS>
@@ -85,6 +87,7 @@ sum_phased_kernel(SrcTable<NSRC> src, char *out, size_t bytes, int kcount, size_
 {
     // tile_bytes <= what kcount iterations cover; where it is less, the lanes beyond it load
     // nothing and store nothing (the tile's buffer descriptor ends there)
+    TCCL_STAMP(0, false);
     constexpr int KMAX = kPhasedVecs / U;
     const size_t off = blockIdx.x * tile_bytes;
     const size_t left = bytes > off ? bytes - off : 0;
@@ -115,6 +118,7 @@ template <class Sum, int NSRC>
 __global__ void __launch_bounds__(kPhasedBlock)
 sum_phased_skewed_kernel(SrcTable<NSRC> src, char *out, size_t bytes, size_t tail_first, size_t numel)
 {
+    TCCL_STAMP(0, false);
     constexpr int KMAX = kPhasedVecs;                                   // one vector per lane per iteration
     constexpr size_t span = static_cast<size_t>(kPhasedBlock) * kVecBytes;
     constexpr size_t region = 2 * KMAX * span;

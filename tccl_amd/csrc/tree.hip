@@ -82,6 +82,7 @@ __device__ __forceinline__ void run_job(const tccl_node_job &j, int kcount)
 template <class Sum, bool FULL>
 __global__ void __launch_bounds__(kPhasedBlock) tree_level_kernel(JobTable jobs, int kcount)
 {
+    TCCL_STAMP(0, false);
     const tccl_node_job &j = jobs.job[blockIdx.y];
     if (j.dst[1] != nullptr)
         run_job<Sum, 2, FULL>(j, kcount);
@@ -98,6 +99,7 @@ constexpr int kCopyU = 4;
 
 __global__ void __launch_bounds__(kPhasedBlock) tree_copy_level_kernel(JobTable jobs, int njobs, int esize)
 {
+    TCCL_STAMP(0, false);
     constexpr size_t span_bytes = static_cast<size_t>(kPhasedBlock) * kCopyU * kVecBytes;
     size_t spans[TCCL_MAX_JOBS];
     size_t total = 0;
@@ -139,6 +141,7 @@ __global__ void __launch_bounds__(kPhasedBlock) tree_copy_level_kernel(JobTable 
                                                        kAuxStoreNt);
         }
     }
+    TCCL_STAMP(3, true);
 }
 
 int launch_level(const tccl_node_job *jobs, int njobs, int dtype, size_t chunk_elems, hipStream_t stream)

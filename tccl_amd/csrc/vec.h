@@ -19,6 +19,43 @@ constexpr int kVecBytes = 16;
 constexpr int kMaxBlock = 512;
 constexpr int kNumXcd = 8;
 
+// Time stamps for measurement builds.  The library itself is built without TCCL_STAMPS and
+// TCCL_STAMP() is nothing there.  benchlib/stamped.hip defines it and includes every source of
+// the library as one translation unit: each workgroup then records the 100 MHz wall clock at
+// four points of its work, in stamp_words[4 * b + slot] for workgroup b (y-major):
+//   slot 0  the workgroup's first instruction            (its first wave)
+//   slot 1  the loads of its first iteration have arrived (latest wave)
+//   slot 2  its last load has arrived and been reduced    (latest wave)
+//   slot 3  its last store has been acknowledged          (latest wave)
+// The host clears the words before a launch and reads them after it.
+#ifdef TCCL_STAMPS
+constexpr int kStampSlots = 4;
+constexpr int kStampMaxWorkgroups = 1 << 16;
+__device__ long long stamp_words[kStampSlots * kStampMaxWorkgroups];
+
+template <int SLOT, bool DRAIN>
+__device__ __forceinline__ void stamp()
+{
+    // SLOT 1 sits inside the read loop: loads of later iterations may still be moved across
+    // it (mask 0x20 = memory reads), the adds that consume this iteration's loads may not
+    __builtin_amdgcn_sched_barrier(SLOT == 1 ? 0x20 : 0);
+    if constexpr (DRAIN) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const long long t = wall_clock64();
+    const size_t b = static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x;
+    if (b < kStampMaxWorkgroups && (threadIdx.x & 63) == 0) {
+        if constexpr (SLOT == 0) {
+            if (threadIdx.x == 0) stamp_words[kStampSlots * b] = t;
+        } else {
+            __hip_atomic_fetch_max(stamp_words + kStampSlots * b + SLOT, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(SLOT == 1 ? 0x20 : 0);
+}
+#define TCCL_STAMP(slot, drain) ::tccl::stamp<slot, drain>()
+#else
+#define TCCL_STAMP(slot, drain) ((void)0)
+#endif
+
 template <bool NT>
 __device__ __forceinline__ u32x4 load_vec(const char *base, size_t vec_index)
 {
@@ -305,8 +342,10 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
             // fp32), which measured 7 % slower there.  (With the 32 KiB tiles of the tree
             // level kernel the barrier measured 1-5 % slower, so it is not used there.)
             if constexpr (PACE) __builtin_amdgcn_sched_barrier(0);
+            if (k == 0) TCCL_STAMP(1, false);
         }
     }
+    TCCL_STAMP(2, false);
 #pragma unroll
     for (int d = 0; d < NDST; ++d) {
         const __amdgpu_buffer_rsrc_t rd = tile_rsrc(dst[d] + tile_off, valid_bytes);
@@ -321,6 +360,7 @@ __device__ __forceinline__ void sum_tile_phased(const char *const (&src)[NSRC], 
             }
         }
     }
+    TCCL_STAMP(3, true);
 }
 
 // Same walk for a plain copy of one source into NDST destinations.
@@ -354,6 +394,7 @@ __device__ __forceinline__ void copy_tile_phased(const char *src, char *const (&
             }
         }
     }
+    TCCL_STAMP(3, true);
 }
 
 // The ragged tail: elements [first, numel), fewer than one vector, one lane each.
