@@ -21,7 +21,8 @@
  *     signal pads.  Where every rank is a process of its own on the same GPU (buffers and pads
  *     exchanged with tccl_ipc_export/open), the same protocol runs between one launch per rank,
  *     as in the reference: tccl_blockwise_barrier(), tccl_double_tree_all_reduce_pipelined_rank(),
- *     tccl_two_shot_all_reduce_rank().
+ *     tccl_two_shot_all_reduce_rank(), and -- with the barrier inside the kernel, as the reference's
+ *     kernels have it -- tccl_all_reduce_sum_rank(), tccl_reduce_scatter_sum_rank(), tccl_all_gather_rank().
  *   - float sums: each bf16 is widened to fp32, accumulated from +0.0f in the order the
  *     sources are given, and rounded once (round-to-nearest-even) on store.  NaN sign
  *     and payload are not specified.
@@ -307,6 +308,44 @@ int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *
 int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void *const *signal_pads,
                                   size_t pad_bytes, int world, int rank, size_t numel, int dtype,
                                   const tccl_pipeline_cfg *cfg, void *stream);
+
+/* The three one-shot collectives as ONE RANK's launch with the reference's barrier inside the
+ * kernel, for ranks that are processes of their own on the same GPU: each replaces one of the
+ * reference's per-rank launches together with the blockwise_barrier its kernel begins with --
+ *   tccl_all_reduce_sum_rank      one_shot_all_reduce_kernel, triton_one_shot_all_reduce_no_128.py:35-64 (barrier :46)
+ *   tccl_reduce_scatter_sum_rank  one_shot_reduce_scatter_kernel, triton_reduce_scatter.py:59-92 (barrier :70, commented out there)
+ *   tccl_all_gather_rank          one_shot_all_gather_kernel, triton_all_gather.py:32-63 (barrier :43)
+ * Workgroup g of this rank's launch meets workgroup g of every other rank's launch (every
+ * rank's buffer is filled, and what was written to it is visible), pulls its tiles from all
+ * `world` buffers (device-scope loads: a peer's producer kernel may end after this kernel
+ * started), writes this rank's `out` -- the results of tccl_all_reduce_sum,
+ * tccl_reduce_scatter_sum and tccl_all_gather, bit for bit -- and meets its peers again: when a
+ * rank's kernel has ended, every rank has read that rank's buffer and it may be refilled (the
+ * trailing barrier the reference lacks).  No barrier launch before or after is needed.
+ * Calling rules: every rank makes the same call with its own `rank` and `out`; bufs and
+ * signal_pads are the same tables in every rank's address space (HOST arrays of `world` device
+ * pointers, peers' entries as opened with tccl_ipc_open); the W launches must be able to run at
+ * the same time (each takes 1/world of the workgroups that fit the GPU, so ranks that share a
+ * stream or a hardware queue can never meet) and must be given the same sizes and the same
+ * cfg->workgroups (the total over all ranks, as always; 0 = chosen by the library, the same in
+ * every rank).  Pads: zero-filled before the first use, left zero-filled by every completed
+ * call, pad_bytes >= 4 * (2 * world + TCCL_PAD_CONTROL_WORDS) (two rows of slots per workgroup:
+ * the leading and the trailing barrier alternate between them, so a flag is never raised over
+ * one that has not been consumed); larger pads allow more workgroups per rank.  The same pads
+ * may serve any sequence of these three calls.  Waits are bounded (cfg->spin_limit, cfg->timeout_flag, the
+ * time-out count in the last word of pad 0): a rank whose peers do not arrive gives up, leaves
+ * `out` unwritten or partly written, and says so.  TCCL_PIPE_DRAW_PLACES does not apply
+ * (TCCL_EINVAL); cfg->lag and cfg->tile_kib are unused.  Preconditions on the sizes as for the
+ * entry points without _rank. */
+int tccl_all_reduce_sum_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes,
+                             int world, int rank, size_t numel, int dtype,
+                             const tccl_pipeline_cfg *cfg, void *stream);
+int tccl_reduce_scatter_sum_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes,
+                                 int world, int rank, size_t numel_total, int dtype,
+                                 const tccl_pipeline_cfg *cfg, void *stream);
+int tccl_all_gather_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes,
+                         int world, int rank, size_t bytes_per_rank,
+                         const tccl_pipeline_cfg *cfg, void *stream);
 
 /* tccl_two_shot_all_reduce() for callers that cannot allocate the signal pads it needs -- code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no

@@ -90,6 +90,9 @@ SIGNATURES = {
     "tccl_signal_pad_timeouts": (_I, [_P, _SZ, ctypes.POINTER(ctypes.c_uint), _P]),
     "tccl_two_shot_all_reduce": (_I, [_PP, _PP, _PP, _SZ, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
     "tccl_two_shot_all_reduce_rank": (_I, [_PP, _P, _PP, _SZ, _I, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
+    "tccl_all_reduce_sum_rank": (_I, [_PP, _P, _PP, _SZ, _I, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
+    "tccl_reduce_scatter_sum_rank": (_I, [_PP, _P, _PP, _SZ, _I, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
+    "tccl_all_gather_rank": (_I, [_PP, _P, _PP, _SZ, _I, _I, _SZ, ctypes.POINTER(PipelineCfg), _P]),
     "tccl_two_shot_all_reduce_static": (_I, [_PP, _PP, _I, _SZ, _I, ctypes.POINTER(PipelineCfg), _P]),
     "tccl_timeout_flag_create": (_I, [ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32))]),
     "tccl_timeout_flag_destroy": (_I, [ctypes.POINTER(ctypes.c_uint32)]),

@@ -17,7 +17,7 @@ from typing import List, Optional
 import torch
 
 from . import _lib, spmd
-from .symm import SymmGroup, rendezvous
+from .symm import RemoteSymmGroup, SymmGroup, rendezvous
 
 _SUM_DTYPES = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}
 
@@ -60,6 +60,30 @@ def _signalling_cfg(group: SymmGroup, cfg: Optional[_lib.PipelineCfg], draw_plac
     return full
 
 
+def _owner_world(group: SymmGroup, what: str, needed: bool = False):
+    """The ``IpcWorld`` of a group whose other buffers belong to other processes, else None.  Such a
+    rank must only ever launch its own work: the per-rank kernels of its world.  ``needed``: ``what``
+    would run every rank's work from this process, so a remote group without a world is refused."""
+    if not isinstance(group, RemoteSymmGroup):
+        return None
+    world = group.world
+    if world is None and needed:
+        raise RuntimeError(f"{what} would run every rank's steps from this process, but the other ranks' buffers "
+                           "belong to other processes: use the IpcWorld the buffer came from")
+    return world
+
+
+def _refuse_remote(group: SymmGroup, what: str) -> None:
+    if isinstance(group, RemoteSymmGroup):
+        raise RuntimeError(f"{what} runs every rank's work from one process; this group's other buffers belong to "
+                           "other processes: every rank calls the per-rank collectives of its IpcWorld instead")
+
+
+def _no_launch_cfg(cfg, what: str) -> None:
+    if cfg is not None:
+        raise ValueError(f"{what}: launch-shape overrides do not apply to the per-rank kernels of an IpcWorld")
+
+
 def _check_out(out: torch.Tensor, shape, like: torch.Tensor) -> torch.Tensor:
     if tuple(out.shape) != tuple(shape) or out.dtype != like.dtype or out.device != like.device \
             or not out.is_contiguous():
@@ -83,6 +107,10 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, out: Optional[torch.Tensor] = N
         symm = rendezvous(tensor)
         symm.group.check_signals()
         output = torch.empty_like(tensor) if out is None else _check_out(out, tensor.shape, tensor)
+        world = _owner_world(symm.group, "one_shot_all_reduce")
+        if world is not None:          # ranks are processes: this rank's launch, barriers inside (the reference's form)
+            _no_launch_cfg(cfg, "one_shot_all_reduce")
+            return world.one_shot_all_reduce(tensor, out=output)
         rc = lib.tccl_all_reduce_sum_ex(symm.buffer_ptrs_host, symm.world_size, output.data_ptr(), tensor.numel(),
                                         dtype, _stream(tensor.device), _cfg_ptr(cfg))
         _lib.check("tccl_all_reduce_sum", rc)
@@ -107,6 +135,10 @@ def one_shot_reduce_scatter(tensor: torch.Tensor, *, out: Optional[torch.Tensor]
             output = torch.empty((per_rank,), dtype=tensor.dtype, device=tensor.device)
         else:
             output = _check_out(out, (per_rank,), tensor)
+        owner = _owner_world(symm.group, "one_shot_reduce_scatter")
+        if owner is not None:
+            _no_launch_cfg(cfg, "one_shot_reduce_scatter")
+            return owner.reduce_scatter(tensor, out=output)
         rc = lib.tccl_reduce_scatter_sum_ex(symm.buffer_ptrs_host, world, rank, output.data_ptr(), tensor.numel(),
                                             dtype, _stream(tensor.device), _cfg_ptr(cfg))
         _lib.check("tccl_reduce_scatter_sum", rc)
@@ -133,6 +165,10 @@ def one_shot_all_gather(tensor: torch.Tensor, world_size: Optional[int] = None, 
             output = torch.empty((world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
         else:
             output = _check_out(out, (world_size, *tensor.shape), tensor)
+        owner = _owner_world(symm.group, "one_shot_all_gather")
+        if owner is not None:
+            _no_launch_cfg(cfg, "one_shot_all_gather")
+            return owner.all_gather(tensor, out=output)
         rc = lib.tccl_all_gather_ex(symm.buffer_ptrs_host, world_size, output.data_ptr(), nbytes,
                                     _stream(tensor.device), _cfg_ptr(cfg))
         _lib.check("tccl_all_gather", rc)
@@ -157,6 +193,9 @@ def two_shot_all_reduce(tensor: torch.Tensor) -> torch.Tensor:
         symm.group.check_signals()
         world = symm.world_size
         assert tensor.numel() % (_vec_elems(tensor) * world) == 0, "The number of elements must be 128-bit aligned."
+        owner = _owner_world(symm.group, "two_shot_all_reduce", needed=True)
+        if owner is not None:          # in place there: every buffer ends up holding the result
+            return owner.two_shot_all_reduce(tensor)
         per_rank = tensor.numel() // world
         shares = torch.empty((world, per_rank), dtype=tensor.dtype, device=tensor.device)
         output = torch.empty_like(tensor)
@@ -175,6 +214,11 @@ def all_reduce(tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
     ``"auto"``.  With every buffer in the same HBM the one-shot kernel moves the fewest bytes
     ((W+1)N against (W+3)N for two-shot and more for the tree), so ``"auto"`` is one-shot at
     every size; the other two exist for what they model across GPUs."""
+    if algorithm not in ("auto", "one_shot", "two_shot", "double_tree"):
+        raise ValueError(f"unknown all-reduce algorithm {algorithm!r}")
+    owner = _owner_world(rendezvous(tensor).group, "all_reduce")
+    if owner is not None:              # ranks are processes: there the three really differ, by size
+        return owner.all_reduce(tensor, algorithm)
     if algorithm in ("auto", "one_shot"):
         return one_shot_all_reduce(tensor)
     if algorithm == "two_shot":
@@ -258,6 +302,13 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
     when ``fused`` is None too, where it is the fastest of the three."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
+    owner = _owner_world(rendezvous(tensor).group, "double_tree_all_reduce", needed=True)
+    if owner is not None:
+        # ranks are processes: this rank's own launch of the pipelined kernel between barriers; running
+        # the node steps of all ranks from here would reduce the mapped buffers W times over
+        if fused or pipelined is False:
+            raise ValueError("double_tree_all_reduce on an IpcWorld buffer runs the per-rank pipelined kernel only")
+        return owner.double_tree_all_reduce(tensor, chunk_elems=chunk_elems)
     if spmd.current_rank() is not None:
         # W rank threads arrive together: one of them runs the collective for everybody,
         # the others pick their output up once it has been enqueued.
@@ -301,6 +352,7 @@ def double_tree_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, 
     run instead of taking them from their hardware index; the launch then makes progress
     however few of its workgroups are resident at once (for use beside other kernels on the
     same GPU), at up to 15 % of the speed on large inputs."""
+    _refuse_remote(group, "double_tree_all_reduce_world")
     like = group.tensors[0].reshape(-1)
     if numel is not None:
         like = like[:numel]
@@ -337,6 +389,7 @@ def two_shot_all_reduce_world(group: SymmGroup, numel: Optional[int] = None, *, 
     Shot 1 reduces each rank's share, the reference's blockwise barrier
     (triton_barrier.py:39-142) separates it from shot 2, which gathers the other shares.
     ``draw_places``: as for ``double_tree_all_reduce_world``."""
+    _refuse_remote(group, "two_shot_all_reduce_world")
     like = group.tensors[0].reshape(-1)
     if numel is not None:
         like = like[:numel]
@@ -368,6 +421,7 @@ class DoubleTreePlan:
     the same buffers and is small enough to be bound by its launches."""
 
     def __init__(self, group: SymmGroup, numel: Optional[int] = None, *, chunk_elems: int = 0):
+        _refuse_remote(group, "DoubleTreePlan")
         like = group.tensors[0].reshape(-1)
         if numel is not None:
             like = like[:numel]

@@ -45,6 +45,9 @@ namespace tccl {
 
 constexpr int kPipeMaxWorld = TCCL_MAX_WORLD;
 constexpr uint32_t kPipeDefaultSpins = 1u << 21;
+// Most workgroups per compute unit a grid whose workgroups wait for each other may have (see
+// resident_for).
+constexpr int kMaxSignallingPerUnit = 6;
 
 // Two signalling kernels that overlap on one GPU could each hold part of the workgroup slots
 // and (with places bound by hardware index) starve each other until their waits expire; with
@@ -476,21 +479,27 @@ static size_t workgroups_per_rank(size_t units, size_t most, int world, bool tie
     return best;
 }
 
-// Workgroups of a kernel that can be resident at once on the current device.
+// Workgroups of kernel `k` that fit the device at once.
+// The hardware hands a grid's workgroups to the 8 XCDs round-robin and, inside an XCD, to its
+// 32 compute units round-robin (read back from the hardware-id register of every workgroup
+// of grids of 4 and 6 per unit: every unit got exactly its share), so a grid of
+// per_cu * units workgroups is resident as a whole once earlier work has left the units.
+// With the registers the signalling kernels need that is 2 to 5 per unit.  Never more than 6:
+// a signalling grid of 8 per unit once timed out for a reason that was never established, so
+// that shape stays unreachable whatever a kernel's register use becomes.
+template <class K>
+static int resident_for(K kernel)
+{
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kPhasedBlock, 0) != hipSuccess || per_cu < 1) return 0;
+    if (per_cu > kMaxSignallingPerUnit) per_cu = kMaxSignallingPerUnit;
+    return per_cu * compute_units();
+}
+
 template <class Sum, int VECS>
 static int resident_workgroups()
 {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, tree_pipelined_kernel<Sum, VECS>, kPhasedBlock, 0) !=
-            hipSuccess ||
-        per_cu < 1)
-        return 0;
-    // The hardware hands a grid's workgroups to the 8 XCDs round-robin and, inside an XCD, to its
-    // 32 compute units round-robin (read back from the hardware-id register of every workgroup
-    // of grids of 4 and 6 per unit: every unit got exactly its share), so a grid of
-    // per_cu * units workgroups is resident as a whole once earlier work has left the units.
-    // With the registers these kernels need (94 to 215 per lane) that is 5, 4 or 2 per unit.
-    return per_cu * compute_units();
+    return resident_for(tree_pipelined_kernel<Sum, VECS>);
 }
 
 template <class Sum, int VECS>
@@ -843,13 +852,7 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, cons
 {
     static std::once_flag once;
     static int resident = 0;
-    std::call_once(once, [] {
-        int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, two_shot_kernel<Sum, W>, kPhasedBlock, 0) ==
-                hipSuccess &&
-            per_cu >= 1)
-            resident = per_cu * compute_units();
-    });
+    std::call_once(once, [] { resident = resident_for(two_shot_kernel<Sum, W>); });
     if (resident < W) return hip_code(hipErrorLaunchOutOfResources);
     constexpr size_t tile_bytes = static_cast<size_t>(kPhasedBlock) * kTwoShotVecs * kVecBytes;
     const size_t tiles = (a.share_bytes + tile_bytes - 1) / tile_bytes;
@@ -986,6 +989,261 @@ extern "C" int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void 
     if (nothing) return TCCL_OK;
     return two_shot_launch(bufs, out ? outs : nullptr, pads, pad_bytes, world, numel, dtype, cfg, nullptr,
                            static_cast<hipStream_t>(stream), rank);
+}
+
+// ------------------------------------------------------------------ one-shot collectives, one launch per rank
+namespace tccl {
+
+// The reference's one-shot kernels begin with blockwise_barrier inside the kernel
+// (triton_one_shot_all_reduce_no_128.py:46, triton_all_gather.py:43, commented at
+// triton_reduce_scatter.py:70): every rank launches its own kernel, whose workgroup g first
+// meets workgroup g of every other rank's kernel ("your buffer is filled") and then pulls
+// from all W buffers.  Here the same as one launch per rank over IPC-mapped buffers and pads,
+// plus the barrier the reference lacks at the end ("I have read your buffer, refill it").
+//
+// The two barriers of a call use different rows of slots: row g for the leading one, row
+// wgs + g for the trailing one.  A rank raises its flag for barrier k+1 of a row only after
+// it has passed barrier k of the other row, which its peer raises only after it has lowered
+// the flag of barrier k of this row -- so a flag is never raised over one that has not been
+// consumed, within a call and from call to call, without the sender having to wait for the
+// slot to be lowered.
+struct RankArgs {
+    const char *src[kPipeMaxWorld]; // sums: every rank's buffer at the first byte this launch reduces; gather: every rank's buffer
+    char *out;
+    uint32_t *pad[kPipeMaxWorld];
+    size_t bytes; // sums: bytes to reduce; gather: bytes per rank
+    uint32_t spin_limit;
+    int world, rank, wgs;
+    uint32_t *ctl;    // control words at the end of pad 0 (time-outs)
+    uint32_t *report; // optional host word set to 1 when a wait expires
+};
+
+// triton_barrier.py:39-142 between workgroup g of this launch and workgroup g of every other
+// rank's launch, on row `row` of the pads.
+__device__ __forceinline__ bool rank_barrier(const RankArgs &a, uint32_t row, int *lds_ok)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const int lane = threadIdx.x;
+    if (lane < a.world && lane != a.rank) {
+        const uint32_t base = row * static_cast<uint32_t>(a.world);
+        __hip_atomic_store(a.pad[lane] + base + a.rank, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t *mine = a.pad[a.rank] + base + lane;
+        uint32_t polls = 0;
+        bool ok = true;
+        while (__hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+            if (++polls >= a.spin_limit) {
+                ok = false;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        if (ok)
+            __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+            report_timeout(a.ctl, a.report);
+        if (!ok) *lds_ok = 0;
+    }
+    __syncthreads();
+    return *lds_ok != 0;
+}
+
+// 16 KiB tiles, as in the two-shot kernel: a rank has 1/W of the GPU's workgroup slots, and
+// small tiles spread a small input over all of them.
+constexpr int kRankVecs = 4;
+
+// All-reduce (bytes = the whole buffer) and reduce-scatter (src offset to this rank's share,
+// bytes = the share): out = sum over the W sources in rank order.  Loads are device-scope: a
+// peer's producer kernel may have finished after this kernel started, so nothing read here
+// may come from a line this XCD's L2 already holds.
+template <class Sum, int W>
+__global__ void __launch_bounds__(kPhasedBlock) sum_rank_kernel(RankArgs a)
+{
+    __shared__ int lds_ok;
+    constexpr int VECS = kRankVecs;
+    constexpr int U = PhasedUnroll<W>::value < VECS ? PhasedUnroll<W>::value : VECS;
+    constexpr int KMAX = VECS / U;
+    constexpr uint32_t span = kPhasedBlock * U * kVecBytes;
+    constexpr uint32_t tile_bytes = kPhasedBlock * VECS * kVecBytes;
+    const uint32_t g = blockIdx.x, G = a.wgs;
+    if (threadIdx.x == 0) lds_ok = 1;
+    if (W > 1 && !rank_barrier(a, g, &lds_ok)) return;
+
+    const char *src[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) src[i] = a.src[i];
+    const char *const(&csrc)[W] = src;
+    char *const dst[1] = {a.out};
+    for (size_t t = static_cast<size_t>(g) * tile_bytes; t < a.bytes; t += static_cast<size_t>(G) * tile_bytes) {
+        const size_t left = a.bytes - t;
+        const uint32_t valid = left < tile_bytes ? static_cast<uint32_t>(left) : tile_bytes;
+        if (valid == tile_bytes)
+            sum_tile_phased<Sum, W, 1, U, KMAX, true, false, kAuxLoadDevice>(csrc, dst, t, valid, KMAX);
+        else
+            sum_tile_phased<Sum, W, 1, U, KMAX, false, false, kAuxLoadDevice>(csrc, dst, t, valid,
+                                                                              static_cast<int>((valid + span - 1) / span));
+    }
+    if (W > 1) (void)rank_barrier(a, G + g, &lds_ok);
+}
+
+// All-gather: out[s] = rank s's buffer for every s, starting at a different peer per rank.
+__global__ void __launch_bounds__(kPhasedBlock) gather_rank_kernel(RankArgs a)
+{
+    __shared__ int lds_ok;
+    constexpr int VECS = kRankVecs;
+    constexpr uint32_t span = kPhasedBlock * 4 * kVecBytes;
+    constexpr uint32_t tile_bytes = kPhasedBlock * VECS * kVecBytes;
+    const uint32_t g = blockIdx.x, G = a.wgs;
+    if (threadIdx.x == 0) lds_ok = 1;
+    if (a.world > 1 && !rank_barrier(a, g, &lds_ok)) return;
+    for (int i = 0; i < a.world; ++i) {
+        const int s = (a.rank + i) % a.world;
+        char *const dst[1] = {a.out + static_cast<size_t>(s) * a.bytes};
+        for (size_t t = static_cast<size_t>(g) * tile_bytes; t < a.bytes; t += static_cast<size_t>(G) * tile_bytes) {
+            const size_t left = a.bytes - t;
+            const uint32_t valid = left < tile_bytes ? static_cast<uint32_t>(left) : tile_bytes;
+            copy_tile_phased<1, 4, VECS / 4, kAuxLoadDevice>(a.src[s], dst, t, valid, static_cast<int>((valid + span - 1) / span));
+        }
+    }
+    if (a.world > 1) (void)rank_barrier(a, G + g, &lds_ok);
+}
+
+// Every rank computes the same count from the same arguments: its launch takes 1/W of the
+// workgroups that fit the device, so that all W launches can be resident together.
+template <class K>
+static int launch_rank_kernel(K kernel, int resident, RankArgs a, size_t tiles, int wgs_wanted, size_t pad_words,
+                              hipStream_t s)
+{
+    if (resident < a.world) return hip_code(hipErrorLaunchOutOfResources);
+    // two rows of slots (leading and trailing barrier), one slot per (workgroup, sender)
+    const size_t fit = (pad_words - kCtlWords) / (2 * static_cast<size_t>(a.world));
+    if (fit < 1) return TCCL_EINVAL;
+    size_t most = static_cast<size_t>(resident / a.world);
+    if (most > fit) most = fit;
+    size_t per_rank;
+    if (wgs_wanted > 0) { // as everywhere in tccl_pipeline_cfg: the total over all ranks
+        per_rank = static_cast<size_t>(wgs_wanted) / static_cast<size_t>(a.world);
+        if (per_rank > most) per_rank = most;
+        if (per_rank > tiles) per_rank = tiles;
+    } else {
+        per_rank = workgroups_per_rank(tiles, most, a.world, false);
+    }
+    if (per_rank < 1) per_rank = 1;
+    a.wgs = static_cast<int>(per_rank);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(per_rank)), dim3(kPhasedBlock), 0, s, a);
+    return hip_code(hipGetLastError());
+}
+
+template <class Sum, int W>
+static int launch_sum_rank_w(const RankArgs &a, size_t tiles, int wgs, size_t pad_words, hipStream_t s)
+{
+    // asked once per kernel: the answer depends on the kernel's register use only
+    static std::once_flag once;
+    static int resident = 0;
+    std::call_once(once, [] { resident = resident_for(sum_rank_kernel<Sum, W>); });
+    return launch_rank_kernel(sum_rank_kernel<Sum, W>, resident, a, tiles, wgs, pad_words, s);
+}
+
+template <class Sum>
+static int launch_sum_rank(const RankArgs &a, size_t tiles, int wgs, size_t pad_words, hipStream_t s)
+{
+    switch (a.world) {
+    case 1: return launch_sum_rank_w<Sum, 1>(a, tiles, wgs, pad_words, s);
+    case 2: return launch_sum_rank_w<Sum, 2>(a, tiles, wgs, pad_words, s);
+    case 3: return launch_sum_rank_w<Sum, 3>(a, tiles, wgs, pad_words, s);
+    case 4: return launch_sum_rank_w<Sum, 4>(a, tiles, wgs, pad_words, s);
+    case 5: return launch_sum_rank_w<Sum, 5>(a, tiles, wgs, pad_words, s);
+    case 6: return launch_sum_rank_w<Sum, 6>(a, tiles, wgs, pad_words, s);
+    case 7: return launch_sum_rank_w<Sum, 7>(a, tiles, wgs, pad_words, s);
+    case 8: return launch_sum_rank_w<Sum, 8>(a, tiles, wgs, pad_words, s);
+    default: return TCCL_EINVAL;
+    }
+}
+
+// Checks and argument block shared by the three entry points.  `first_byte`: where in every
+// buffer this launch starts to read.
+static int rank_args(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes, int world, int rank,
+                     size_t first_byte, size_t bytes, const tccl_pipeline_cfg *cfg, RankArgs *a)
+{
+    if (bufs == nullptr || out == nullptr || signal_pads == nullptr || world < 1 || world > TCCL_MAX_WORLD || rank < 0 ||
+        rank >= world)
+        return TCCL_EINVAL;
+    if (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) return TCCL_EINVAL; // places are fixed by the rank's own launch
+    if (pad_bytes % 16 != 0 || pad_bytes < (2 * static_cast<size_t>(world) + kCtlWords) * sizeof(uint32_t)) return TCCL_EINVAL;
+    if (!aligned16(out)) return TCCL_EALIGN;
+    *a = RankArgs{};
+    for (int r = 0; r < world; ++r) {
+        if (bufs[r] == nullptr || signal_pads[r] == nullptr) return TCCL_EINVAL;
+        if (!aligned16(bufs[r]) || !aligned16(signal_pads[r])) return TCCL_EALIGN;
+        a->src[r] = static_cast<const char *>(bufs[r]) + first_byte;
+        a->pad[r] = static_cast<uint32_t *>(signal_pads[r]);
+    }
+    a->out = static_cast<char *>(out);
+    a->bytes = bytes;
+    a->spin_limit = (cfg && cfg->spin_limit > 0) ? cfg->spin_limit : kPipeDefaultSpins;
+    a->world = world;
+    a->rank = rank;
+    a->ctl = a->pad[0] + pad_bytes / sizeof(uint32_t) - kCtlWords;
+    a->report = cfg ? cfg->timeout_flag : nullptr;
+    return TCCL_OK;
+}
+
+static int sum_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes, int world, int rank,
+                    size_t first_elem, size_t numel, int dtype, const tccl_pipeline_cfg *cfg, void *stream)
+{
+    const int esize = dtype_size(dtype);
+    if (esize == 0) return TCCL_EINVAL;
+    if ((numel * esize) % kVecBytes != 0 || (first_elem * esize) % kVecBytes != 0) return TCCL_EALIGN;
+    RankArgs a;
+    const int rc = rank_args(bufs, out, signal_pads, pad_bytes, world, rank, first_elem * esize, numel * esize, cfg, &a);
+    if (rc != TCCL_OK) return rc;
+    // an empty input still meets the peers: the barriers are the collective's ordering
+    constexpr size_t tile_bytes = static_cast<size_t>(kPhasedBlock) * kRankVecs * kVecBytes;
+    size_t tiles = (a.bytes + tile_bytes - 1) / tile_bytes;
+    if (tiles < 1) tiles = 1;
+    const int wgs = cfg ? cfg->workgroups : 0;
+    const size_t pad_words = pad_bytes / sizeof(uint32_t);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == TCCL_BF16 ? launch_sum_rank<Bf16Sum>(a, tiles, wgs, pad_words, s)
+                              : launch_sum_rank<F32Sum>(a, tiles, wgs, pad_words, s);
+}
+
+} // namespace tccl
+
+extern "C" int tccl_all_reduce_sum_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes,
+                                        int world, int rank, size_t numel, int dtype, const tccl_pipeline_cfg *cfg,
+                                        void *stream)
+{
+    return sum_rank(bufs, out, signal_pads, pad_bytes, world, rank, 0, numel, dtype, cfg, stream);
+}
+
+extern "C" int tccl_reduce_scatter_sum_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes,
+                                            int world, int rank, size_t numel_total, int dtype,
+                                            const tccl_pipeline_cfg *cfg, void *stream)
+{
+    if (world < 1 || world > TCCL_MAX_WORLD || rank < 0 || rank >= world) return TCCL_EINVAL;
+    // every rank's share is the same whole number of vectors (triton_reduce_scatter.py:101-104)
+    if (numel_total % static_cast<size_t>(world) != 0) return TCCL_EALIGN;
+    const size_t per_rank = numel_total / static_cast<size_t>(world);
+    return sum_rank(bufs, out, signal_pads, pad_bytes, world, rank, static_cast<size_t>(rank) * per_rank, per_rank, dtype,
+                    cfg, stream);
+}
+
+extern "C" int tccl_all_gather_rank(void *const *bufs, void *out, void *const *signal_pads, size_t pad_bytes, int world,
+                                    int rank, size_t bytes_per_rank, const tccl_pipeline_cfg *cfg, void *stream)
+{
+    if (bytes_per_rank % kVecBytes != 0) return TCCL_EALIGN;
+    RankArgs a;
+    const int rc = rank_args(bufs, out, signal_pads, pad_bytes, world, rank, 0, bytes_per_rank, cfg, &a);
+    if (rc != TCCL_OK) return rc;
+    constexpr size_t tile_bytes = static_cast<size_t>(kPhasedBlock) * kRankVecs * kVecBytes;
+    size_t tiles = (a.bytes + tile_bytes - 1) / tile_bytes;
+    if (tiles < 1) tiles = 1;
+    static std::once_flag once;
+    static int resident = 0;
+    std::call_once(once, [] { resident = resident_for(gather_rank_kernel); });
+    return launch_rank_kernel(gather_rank_kernel, resident, a, tiles, cfg ? cfg->workgroups : 0,
+                              pad_bytes / sizeof(uint32_t), static_cast<hipStream_t>(stream));
 }
 
 // ------------------------------------------------------------------ the entry point that allocates nothing

@@ -64,11 +64,15 @@ class IpcWorld:
         self._tree_pads = {}                  # pad size -> table of all ranks' pads for kernels that signal inside a launch
         self._count = 0
         self._host_barriers = 0
+        self._epoch = 0                       # resets so far: time-outs are published per epoch
         self._flag = ctypes.POINTER(ctypes.c_uint32)()
         _lib.check("tccl_timeout_flag_create", self.lib.tccl_timeout_flag_create(ctypes.byref(self._flag)))
         # signal pads: one per rank, every rank maps all of them
         self._pad_ptrs = self._exchange(self._alloc(self.PAD_BYTES), "pad")
         self._pad_array = _lib.ptr_array(self._pad_ptrs)
+        # ... and the pads of the one-shot kernels that carry their barriers themselves, so that a rank's
+        # first collective never has to wait on the host for a peer that is late
+        self._kernel_pads(self.ONE_SHOT_PAD_BYTES)
 
     @classmethod
     def from_env(cls, device="cuda:0", timeout_s: float = 60.0) -> "IpcWorld":
@@ -139,7 +143,7 @@ class IpcWorld:
         own = self._alloc(max(nbytes, 16))
         ptrs = self._exchange(own, "buf")
         tensor = _as_tensor(own, nbytes, self.device).view(dtype)
-        symm.register_remote(tensor, self.rank, ptrs)
+        symm.register_remote(tensor, self.rank, ptrs, world=self)
         self._tables[own] = (ptrs, nbytes, dtype)
         return tensor
 
@@ -224,23 +228,127 @@ class IpcWorld:
         ``one_shot_all_reduce``.  The element count must be a multiple of W vectors."""
         return self._own_launch("tccl_two_shot_all_reduce_rank", tensor, self.TWO_SHOT_PAD_BYTES, (), cfg)
 
+    # Signal pad size of the one-shot kernels: two rows of slots for up to 512 workgroups per rank.
+    ONE_SHOT_PAD_BYTES = 4 * (2 * 8 * 512 + 288)
+
+    def _one_shot(self, name: str, tensor: torch.Tensor, out: torch.Tensor, size_arg: int, with_dtype: bool,
+                  cfg: Optional[_lib.PipelineCfg]) -> torch.Tensor:
+        ptrs, _, dtype = self._tables[self._base(tensor)]
+        pads = self._kernel_pads(self.ONE_SHOT_PAD_BYTES)
+        use = _lib.PipelineCfg()
+        if cfg is not None:
+            ctypes.memmove(ctypes.byref(use), ctypes.byref(cfg), ctypes.sizeof(use))
+        use.timeout_flag = self._flag
+        stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        args = [_lib.ptr_array(ptrs), out.data_ptr(), pads, self.ONE_SHOT_PAD_BYTES, self.world_size, self.rank, size_arg]
+        if with_dtype:
+            args.append({torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype])
+        _lib.check(name, getattr(self.lib, name)(*args, ctypes.byref(use), stream))
+        return out
+
+    def _base(self, tensor: torch.Tensor) -> int:
+        """Address of the symmetric buffer ``tensor`` is (a prefix view of)."""
+        base = tensor.data_ptr()
+        if base not in self._tables:
+            raise RuntimeError("tensor does not come from this world's empty() (or is not a view from its first element)")
+        if not tensor.is_contiguous():
+            raise RuntimeError("a collective must be given a contiguous view")
+        return base
+
+    def one_shot_all_reduce(self, tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+                            cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+        """``one_shot_all_reduce`` the way the reference's kernel runs it (triton_one_shot_all_reduce_no_128.py:35-64):
+        this rank's ONE launch, which meets the peers' launches in ``blockwise_barrier`` first (:46), sums all
+        W buffers in rank order into a fresh output, and meets the peers again before it ends (so the buffers
+        may be refilled as soon as the call's kernel is done).  Collective: every rank calls it."""
+        assert tensor.dtype in (torch.bfloat16, torch.float32), "Only bfloat16 (and float32) is supported for now."
+        assert tensor.numel() % (16 // tensor.element_size()) == 0, "The number of elements must be 128-bit aligned."
+        output = torch.empty_like(tensor) if out is None else out
+        return self._one_shot("tccl_all_reduce_sum_rank", tensor, output, tensor.numel(), True, cfg)
+
+    def reduce_scatter(self, tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+                       cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+        """``one_shot_reduce_scatter`` as one launch of this rank with the barriers inside the kernel
+        (triton_reduce_scatter.py:59-92; the reference has its leading barrier commented out, :70)."""
+        assert tensor.dtype in (torch.bfloat16, torch.float32), "Only bfloat16 (and float32) is supported for now."
+        assert tensor.numel() % ((16 // tensor.element_size()) * self.world_size) == 0, \
+            "The number of elements must be 128-bit aligned."
+        per_rank = tensor.numel() // self.world_size
+        output = torch.empty((per_rank,), dtype=tensor.dtype, device=tensor.device) if out is None else out
+        return self._one_shot("tccl_reduce_scatter_sum_rank", tensor, output, tensor.numel(), True, cfg)
+
+    def all_gather(self, tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+                   cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+        """``one_shot_all_gather`` as one launch of this rank with the barriers inside the kernel
+        (triton_all_gather.py:32-63, leading barrier :43)."""
+        nbytes = tensor.numel() * tensor.element_size()
+        assert nbytes % 16 == 0, "The number of elements must be 128-bit aligned."
+        if out is None:
+            out = torch.empty((self.world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
+        return self._one_shot("tccl_all_gather_rank", tensor, out, nbytes, False, cfg)
+
+    # All-reduce by size, measured with 8 processes on one MI355X (python -m tccl_amd.launch
+    # --nproc-per-node 8 benchlib/ipc_forms.py, us per collective, one-shot / two-shot / double tree):
+    # see ONE_SHOT_MAX_BYTES below.  Across GPUs the one-shot form moves (W-1) whole buffers per rank
+    # over the links and the thresholds would sit far lower; on one GPU they are what was measured.
+    ONE_SHOT_MAX_BYTES = 1 << 62
+
+    def all_reduce(self, tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
+        """All-reduce of this rank's buffer by the named algorithm -- ``"one_shot"`` (fresh output, buffers
+        untouched), ``"two_shot"`` or ``"double_tree"`` (both in place: every buffer ends up holding the
+        result, which is also returned) -- or ``"auto"``: the fastest of the three for the buffer's size."""
+        if algorithm == "auto":
+            nbytes = tensor.numel() * tensor.element_size()
+            vec = 16 // tensor.element_size()
+            algorithm = "one_shot"
+            if nbytes > self.ONE_SHOT_MAX_BYTES and tensor.numel() % (vec * self.world_size) == 0:
+                algorithm = "two_shot"
+        if algorithm == "one_shot":
+            return self.one_shot_all_reduce(tensor)
+        if algorithm == "two_shot":
+            return self.two_shot_all_reduce(tensor)
+        if algorithm == "double_tree":
+            return self.double_tree_all_reduce(tensor)
+        raise ValueError(f"unknown all-reduce algorithm {algorithm!r}")
+
+    def _peer_timeouts(self) -> List[int]:
+        """Ranks that have published an expired wait since the last reset."""
+        prefix = f"timeout{self._epoch}.rank"
+        try:
+            return sorted(int(n[len(prefix):]) for n in os.listdir(self.directory) if n.startswith(prefix))
+        except OSError:
+            return []
+
     def check(self) -> None:
-        """Synchronise and raise if a barrier wait expired (a peer never arrived)."""
+        """Synchronise and raise if a wait of this rank expired (a peer never arrived at a barrier, or at a
+        wait inside a collective's kernel), or if a peer has reported one since the last ``reset()``: that
+        collective's results are partial on some rank.  Every rank should then call ``reset()``."""
         torch.cuda.synchronize(self.device)
         if self._flag[0] != 0:
             self._flag[0] = 0
+            self._publish(f"timeout{self._epoch}.rank{self.rank}", b"1")
             raise _lib.TcclError("tccl_blockwise_barrier", _lib.TCCL_ETIMEOUT,
                                  "a peer did not reach the barrier in time (or a wait inside a collective's kernel expired)")
+        peers = [r for r in self._peer_timeouts() if r != self.rank]
+        if peers:
+            raise _lib.TcclError("a collective of this world", _lib.TCCL_ETIMEOUT,
+                                 f"rank(s) {peers} reported an expired wait: results since the last check may be "
+                                 "partial; every rank must call reset()")
 
     def reset(self) -> None:
-        """Collective: bring the signal pads back to zero after a barrier wait expired (a barrier that
-        gave up leaves flags standing).  Every rank calls it; the ranks meet on the host before and
+        """Collective: bring every signal pad of this world back to zero after a wait expired (a barrier
+        or a signalling kernel that gave up leaves flags standing).  Every rank calls it; the ranks meet on the host before and
         after, so no barrier kernel is running while the pads are cleared."""
         torch.cuda.synchronize(self.device)
         self.host_barrier()
         _as_tensor(self._pad_ptrs[self.rank], self.PAD_BYTES, self.device).zero_()
+        # the pads of the kernels that signal inside a launch, control words included: a wait that
+        # expired there leaves flags standing that the next collective would take for its own
+        for nbytes, table in self._tree_pads.items():
+            _as_tensor(table[self.rank], nbytes, self.device).zero_()
         torch.cuda.synchronize(self.device)
         self._flag[0] = 0
+        self._epoch += 1
         self.host_barrier()
 
     def close(self) -> None:

@@ -143,10 +143,10 @@ def register(tensors: Sequence[torch.Tensor]) -> SymmGroup:
 class RemoteSymmGroup(SymmGroup):
     """A group of which this process owns one buffer; the other ranks' buffers belong to other
     processes and are known by the addresses they are mapped at here (``tccl_amd.ipc``).  Serves
-    the per-rank collectives (all-reduce, reduce-scatter, all-gather), which need the address
-    table, the rank and the world size only."""
+    the per-rank collectives only; anything that would run other ranks' work from this process
+    (the ``*_world`` functions, the in-process double tree) refuses such a group."""
 
-    def __init__(self, own: torch.Tensor, rank: int, buffer_ptrs: Sequence[int]):   # noqa: super().__init__ not called
+    def __init__(self, own: torch.Tensor, rank: int, buffer_ptrs: Sequence[int], world=None):   # noqa: super().__init__ not called
         if not own.is_contiguous() or int(own.data_ptr()) != int(buffer_ptrs[rank]):
             raise ValueError("the own buffer must be the whole allocation at buffer_ptrs[rank]")
         self.tensors = [own]
@@ -161,6 +161,12 @@ class RemoteSymmGroup(SymmGroup):
         self._signal_pad_array = None
         self._timeout_flag = None
         self.own_rank = rank
+        # the IpcWorld the buffer came from: it owns the signal pads the per-rank kernels meet through
+        self._world = weakref.ref(world) if world is not None else None
+
+    @property
+    def world(self):
+        return self._world() if self._world is not None else None
 
     def tensor(self, rank: int) -> torch.Tensor:
         if rank != self.own_rank:
@@ -168,10 +174,12 @@ class RemoteSymmGroup(SymmGroup):
         return self.tensors[0]
 
 
-def register_remote(own: torch.Tensor, rank: int, buffer_ptrs: Sequence[int]) -> RemoteSymmGroup:
+def register_remote(own: torch.Tensor, rank: int, buffer_ptrs: Sequence[int], world=None) -> RemoteSymmGroup:
     """Declare that ``own`` is rank ``rank``'s buffer of a symmetric allocation whose other buffers
-    live in other processes and are mapped here at ``buffer_ptrs`` (rank order)."""
-    group = RemoteSymmGroup(own, rank, buffer_ptrs)
+    live in other processes and are mapped here at ``buffer_ptrs`` (rank order).  ``world``: the
+    ``IpcWorld`` the buffers were exchanged through; with it the reference-named wrappers run the
+    per-rank kernels that carry their barriers themselves."""
+    group = RemoteSymmGroup(own, rank, buffer_ptrs, world)
     _registry[int(own.data_ptr())] = (weakref.ref(group), rank)
     own._tccl_group = group           # noqa: SLF001
     return group

@@ -28,6 +28,20 @@ DOUBLE_TREE_SHAPES = (("small", 98_760, torch.bfloat16), ("big", 4_194_304, torc
 TWO_SHOT_SHAPES = (("small", 8 * 37, torch.bfloat16), ("big", 8 * 65_537, torch.bfloat16), ("f32", 4 * 20_011, torch.float32))
 
 
+# (name, elements per rank's share, dtype) for the one-shot kernels that carry their barriers themselves:
+# less than one tile in all; many tiles with a ragged last one; fp32; enough tiles for every workgroup of a rank
+ONE_SHOT_SHAPES = (("small", 8 * 5, torch.bfloat16), ("ragged", 8 * 4099, torch.bfloat16), ("f32", 4 * 10_007, torch.float32),
+                   ("big", 8 * 131_072, torch.bfloat16))
+
+
+def fill(t, numel, dtype, seed):
+    torch.manual_seed(seed)
+    if dtype == torch.bfloat16:
+        t.copy_(torch.randn(numel, dtype=dtype))
+    else:
+        t.copy_(torch.rand(numel, dtype=dtype) * 2 - 1)
+
+
 def save(directory, name, rank, t):
     t = t.detach().cpu().contiguous()
     view = {2: torch.int16, 4: torch.int32, 1: torch.int8}[t.element_size()]
@@ -56,6 +70,102 @@ def main():
         print(f"rank {rank}: barrier works after the reset", flush=True)
         world.close()
         return 42 if reported else (0 if rank != 0 else 1)
+
+    if mode == "one_shot_rank":
+        # all-reduce, reduce-scatter and all-gather as ONE launch per rank each, the leading and the
+        # trailing barrier inside the kernel: no barrier launch anywhere, no host barrier between the
+        # rounds -- a rank refills its buffer as soon as its own kernels are done, which is exactly
+        # what the trailing barrier has to make safe
+        for tag, per_rank, dtype in ONE_SHOT_SHAPES:
+            numel = per_rank * world_size
+            t = world.empty(numel, dtype)
+            for round_ in range(2):
+                fill(t, numel, dtype, 100 * round_ + rank)
+                if (round_ + rank) % 3 == 0:
+                    torch.cuda._sleep(2_000_000)          # ranks out of step
+                if round_ == 0:
+                    outs = (world.one_shot_all_reduce(t), world.reduce_scatter(t), world.all_gather(t))
+                else:                                      # the reference's names find the world by themselves
+                    outs = (tccl_amd.one_shot_all_reduce(t), tccl_amd.reduce_scatter(t), tccl_amd.all_gather(t, world_size))
+                for name, o in zip(("all_reduce", "reduce_scatter", "all_gather"), outs):
+                    save(directory, f"rank_{name}_{tag}.{round_}", rank, o)
+            world.check()
+            print(f"rank {rank}: one-shot kernels {tag} done", flush=True)
+        pad = world._kernel_pads(world.ONE_SHOT_PAD_BYTES)
+        own = ipc._as_tensor(pad[rank], world.ONE_SHOT_PAD_BYTES, world.device).view(torch.int32)
+        world.barrier()
+        left = int(own.ne(0).sum())
+        world.check()
+        world.close()
+        if left:
+            print(f"rank {rank}: {left} words of the signal pad are not zero after the collectives", flush=True)
+            return 5
+        return 0
+
+    if mode == "one_shot_missing_peer":
+        # rank 0 starts an all-reduce with a small spin limit and nobody joins: its kernel must end by
+        # itself and the rank must be told; after a collective reset everybody's collectives work
+        numel = 8 * world_size * 1031
+        t = world.empty(numel, torch.bfloat16)
+        reported = False
+        if rank == 0:
+            cfg = tccl_amd._lib.PipelineCfg()
+            cfg.spin_limit = 2000
+            world.one_shot_all_reduce(t, cfg=cfg)
+            try:
+                world.check()
+            except tccl_amd.TcclError as e:
+                print(f"rank 0: reported: {e}", flush=True)
+                reported = True
+        world.reset()
+        for round_ in range(2):
+            fill(t, numel, torch.bfloat16, 100 * round_ + rank)
+            save(directory, f"after_reset.{round_}", rank, world.one_shot_all_reduce(t))
+        world.check()
+        world.close()
+        return 42 if reported else (0 if rank != 0 else 1)
+
+    if mode == "kernel_timeout_reset":
+        # a wait INSIDE a collective's kernel expires on some ranks (rank 1's stream is held back behind
+        # the leading barrier while the others run the two-shot kernel with a small spin limit); the
+        # flags they leave standing in the kernel pads must be gone after reset(), or the next
+        # collective on the same pads would pass its barrier early and return partial sums
+        numel = 8 * world_size * 2053
+        t = world.empty(numel, torch.bfloat16)
+        fill(t, numel, torch.bfloat16, rank)
+        cfg = tccl_amd._lib.PipelineCfg()
+        cfg.spin_limit = 3000 if rank != 1 else 0
+        world.barrier()
+        if rank == 1:
+            torch.cuda._sleep(400_000_000)                # about 0.2 s on the GPU, bounded
+        ptrs = tccl_amd._lib.ptr_array(world._tables[t.data_ptr()][0])
+        pads = world._kernel_pads(world.TWO_SHOT_PAD_BYTES)
+        cfg.timeout_flag = world._flag
+        import ctypes
+        rc = world.lib.tccl_two_shot_all_reduce_rank(ptrs, None, pads, world.TWO_SHOT_PAD_BYTES, world_size, rank, numel, 0,
+                                                     ctypes.byref(cfg), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, rc
+        reported = False
+        try:
+            world.check()
+        except tccl_amd.TcclError as e:
+            print(f"rank {rank}: reported: {e}", flush=True)
+            reported = True
+        world.host_barrier()                              # every rank has looked at its own flag
+        try:
+            world.check()                                 # ... and now also sees what the peers published
+        except tccl_amd.TcclError as e:
+            print(f"rank {rank}: told: {e}", flush=True)
+            reported = True
+        world.reset()
+        for round_ in range(2):
+            fill(t, numel, torch.bfloat16, 100 * (round_ + 1) + rank)
+            out = world.two_shot_all_reduce(t)
+            world.check()
+            save(directory, f"after_kernel_timeout.{round_}", rank, out)
+            world.host_barrier()
+        world.close()
+        return 42 if reported else 1
 
     if mode == "reference_mains":
         # the self-tests at the bottom of the reference's four kernel files, with a process per rank

@@ -112,6 +112,63 @@ def test_two_shot_one_launch_per_rank(world, tmp_path):
                     assert torch.equal(got, want), f"{tag} round {round_} rank {r} {what}"
 
 
+@pytest.mark.parametrize("world", [4, 8])
+def test_one_shot_kernels_with_their_barriers_inside(world, tmp_path):
+    """The reference's form for process-owned ranks (triton_one_shot_all_reduce_no_128.py:46,
+    triton_all_gather.py:43): every rank's all-reduce, reduce-scatter and all-gather is ONE launch that
+    begins with the blockwise barrier and -- beyond the reference -- ends with one.  bf16 and fp32, two
+    rounds per shape with a refill between them and no other synchronisation; against the oracle, bit for bit."""
+    from ipc_rank_program import ONE_SHOT_SHAPES
+    print(f"ipc: one-shot kernels with barriers inside, {world} processes", flush=True)
+    codes, outs = run_ranks(world, tmp_path, "one_shot_rank", timeout=150)
+    assert codes == [0] * world, "\n".join(outs)
+    for tag, per_rank, dtype in ONE_SHOT_SHAPES:
+        numel = per_rank * world
+        bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+        for round_ in range(2):
+            bufs = (seeded_randn(world, numel, seed_base=100 * round_) if dtype == torch.bfloat16
+                    else seeded_uniform(world, numel, seed_base=100 * round_))
+            want = torch_ref.all_reduce(bufs).view(bits)
+            stacked = torch.stack(bufs).view(bits)
+            for r in range(world):
+                got = load(tmp_path, f"rank_all_reduce_{tag}.{round_}", r, dtype).view(bits)
+                assert torch.equal(got, want), f"{tag} round {round_} rank {r}: all-reduce"
+                got = load(tmp_path, f"rank_reduce_scatter_{tag}.{round_}", r, dtype).view(bits)
+                assert torch.equal(got, want[r * per_rank:(r + 1) * per_rank]), f"{tag} round {round_} rank {r}: reduce-scatter"
+                got = load(tmp_path, f"rank_all_gather_{tag}.{round_}", r, dtype).view(bits)
+                assert torch.equal(got, stacked), f"{tag} round {round_} rank {r}: all-gather"
+
+
+def test_one_shot_kernel_with_a_missing_peer_gives_up_and_says_so(tmp_path):
+    """Failure handling forced from the host: rank 0 launches its all-reduce with a small spin limit and
+    no peer ever does.  The kernel ends by itself at its leading barrier, the rank is told, and after a
+    collective reset (which clears the flags it left in the peers' pads) the collective works."""
+    world, numel = 2, 8 * 2 * 1031
+    codes, outs = run_ranks(world, tmp_path, "one_shot_missing_peer", timeout=90)
+    assert codes == [42, 0], "\n".join(outs)
+    assert "expired" in outs[0]
+    for round_ in range(2):
+        want = torch_ref.all_reduce(seeded_randn(world, numel, seed_base=100 * round_)).view(torch.int16)
+        for r in range(world):
+            assert torch.equal(load(tmp_path, f"after_reset.{round_}", r, torch.bfloat16).view(torch.int16), want)
+
+
+def test_reset_clears_the_pads_of_the_signalling_kernels(tmp_path):
+    """A wait inside the two-shot kernel expires on three of four ranks (forced from the host: the fourth
+    rank's stream is held back, the others poll a few thousand times).  They report it, the fourth is told
+    through the rendezvous directory, reset() clears every pad -- the kernels' as well as the barrier's --
+    and the next collectives on the same pads match the oracle."""
+    world, numel = 4, 8 * 4 * 2053
+    codes, outs = run_ranks(world, tmp_path, "kernel_timeout_reset", timeout=120)
+    assert codes == [42] * world, "\n".join(outs)
+    assert sum("reported:" in o for o in outs) >= 1
+    for round_ in range(2):
+        want = torch_ref.all_reduce(seeded_randn(world, numel, seed_base=100 * (round_ + 1))).view(torch.int16)
+        for r in range(world):
+            got = load(tmp_path, f"after_kernel_timeout.{round_}", r, torch.bfloat16).view(torch.int16)
+            assert torch.equal(got, want), f"round {round_} rank {r}"
+
+
 @pytest.mark.parametrize("world", [8, 4])
 def test_reference_self_tests_with_a_process_per_rank(world, tmp_path):
     """The `__main__` self-tests of the reference's kernel files (every rank fills its buffer
