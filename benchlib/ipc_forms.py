@@ -1,0 +1,95 @@
+"""What the collectives cost when every rank is a process of its own on the one GPU, form by form:
+
+    python -m tccl_amd.launch --nproc-per-node 8 benchlib/ipc_forms.py
+
+Per buffer size rank 0 prints the time per collective (HIP events on its own stream, all ranks in
+step: the median and, in brackets, the fastest of 5 blocks of 16 calls after 8 warm-up calls) of
+
+  barrier             tccl_blockwise_barrier alone (one launch per rank)
+  one-shot x3         barrier launch + tccl_all_reduce_sum + barrier launch (three launches per rank)
+  one-shot fused      tccl_all_reduce_sum_rank: one launch per rank, both barriers inside the kernel
+  rs x3 / rs fused    the same two forms of the reduce-scatter
+  ag x3 / ag fused    ... and of the all-gather (every rank contributes 1/W of the buffer size)
+  two-shot x3 / fused barrier + tccl_two_shot_all_reduce_rank + barrier, and the same kernel with
+                      TCCL_PIPE_OWN_BARRIERS: one launch per rank (both in place)
+  tree                barrier + tccl_double_tree_all_reduce_pipelined_rank + barrier (in place)
+
+The in-place forms rescale the buffer before every call so that values stay finite; that small
+kernel is part of their time.  On one GPU the W processes' queues take turns, so these times say how
+the forms compare with each other here, not what they would cost with a GPU per rank."""
+import ctypes
+import os
+import sys
+
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+from tccl_amd import _lib, ipc        # noqa: E402
+
+
+def main() -> int:
+    world = ipc.IpcWorld.from_env()
+    rank, size = world.rank, world.world_size
+    lib = world.lib
+
+    def timed(fn, reps=16, warm=8, blocks=5):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        world.host_barrier()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(blocks + 1)]
+        ev[0].record()
+        for b in range(blocks):
+            for _ in range(reps):
+                fn()
+            ev[b + 1].record()
+        torch.cuda.synchronize()
+        world.check()
+        us = sorted(ev[b].elapsed_time(ev[b + 1]) * 1000 / reps for b in range(blocks))
+        return f"{us[blocks // 2]:.0f} ({us[0]:.0f})"
+
+    if rank == 0:
+        print(f"{size} processes on one GPU; us per collective on rank 0's stream", flush=True)
+        print(f"{'per buffer':>10s} {'barrier':>10s} | {'one-shot x3':>11s} {'fused':>11s} | {'rs x3':>10s} {'fused':>10s} | "
+              f"{'ag x3':>10s} {'fused':>10s} | {'two-shot x3':>11s} {'fused':>11s} | {'tree':>11s}", flush=True)
+    for kib in (64, 1024, 4096, 16384, 65536, 262144):
+        numel = kib << 9
+        t = world.empty(numel, torch.bfloat16)
+        t.copy_(torch.randn(numel, dtype=torch.bfloat16) * 0.01)
+        ptrs = _lib.ptr_array(world._tables[t.data_ptr()][0])
+        out = torch.empty_like(t)
+        share = torch.empty(numel // size, dtype=torch.bfloat16, device=t.device)
+        part = t[: numel // size]                       # all-gather: every rank contributes 1/W of the buffer
+        gathered = torch.empty((size, numel // size), dtype=torch.bfloat16, device=t.device)
+
+        def stream():
+            return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+        def between_barriers(call):
+            def run():
+                world.barrier()
+                assert call() == 0
+                world.barrier()
+            return run
+
+        us = [timed(world.barrier)]
+        us.append(timed(between_barriers(lambda: lib.tccl_all_reduce_sum(ptrs, size, out.data_ptr(), numel, 0, stream()))))
+        us.append(timed(lambda: world.one_shot_all_reduce(t, out=out)))
+        us.append(timed(between_barriers(lambda: lib.tccl_reduce_scatter_sum(ptrs, size, rank, share.data_ptr(), numel, 0, stream()))))
+        us.append(timed(lambda: world.reduce_scatter(t, out=share)))
+        us.append(timed(between_barriers(lambda: lib.tccl_all_gather(ptrs, size, gathered.data_ptr(), part.numel() * 2, stream()))))
+        us.append(timed(lambda: world.all_gather(part, out=gathered)))
+        us.append(timed(lambda: (t.mul_(1.0 / size), world.two_shot_all_reduce(t, own_barriers=False))))
+        us.append(timed(lambda: (t.mul_(1.0 / size), world.two_shot_all_reduce(t))))
+        us.append(timed(lambda: (t.mul_(1.0 / size), world.double_tree_all_reduce(t))) if size in (2, 4, 8) else "-")
+        if rank == 0:
+            label = f"{kib} KiB" if kib < 1024 else f"{kib >> 10} MiB"
+            print(f"{label:>10s} {us[0]:>10s} | {us[1]:>11s} {us[2]:>11s} | {us[3]:>10s} {us[4]:>10s} | "
+                  f"{us[5]:>10s} {us[6]:>10s} | {us[7]:>11s} {us[8]:>11s} | {us[9]:>11s}", flush=True)
+    world.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

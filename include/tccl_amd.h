@@ -220,7 +220,8 @@ int tccl_plan_destroy(tccl_plan *plan);
  *   them zero-filled again.  The last TCCL_PAD_CONTROL_WORDS 32-bit words of pad 0 are control
  *   words (counters from which the workgroups draw their places, and -- the very last word,
  *   at pad_bytes - 4 -- the count of time-outs).
- * Waits are bounded (cfg->spin_limit polls): a workgroup whose signal never comes counts a
+ * Waits are bounded (cfg->spin_limit pauses of about 0.2 us; polls back off from one pause to 128
+ * between two polls while a flag stays away): a workgroup whose signal never comes counts a
  *   time-out and leaves the kernel, and so does everyone who waits for it, so the launch
  *   always ends; the buffers then hold partial results and the pads must be cleared by the
  *   caller.  tccl_signal_pad_timeouts() reads the count (it synchronises the stream); a caller
@@ -247,7 +248,7 @@ int tccl_plan_destroy(tccl_plan *plan);
 typedef struct {
     int workgroups;      /* total workgroups (all ranks); 0 = chosen by the library */
     int lag;             /* 1 + rounds the down-sweep runs behind the up-sweep; 0 = default (1: none) */
-    unsigned spin_limit; /* polls before a wait gives up; 0 = default (about a second) */
+    unsigned spin_limit; /* pauses of about 0.2 us before a wait gives up; 0 = default (about half a second) */
     int tile_kib;        /* a workgroup works a chunk in tiles of 32 (default) or 128 KiB */
     uint32_t *timeout_flag; /* NULL, or a device-visible 32-bit word (pinned host memory, e.g. from
                                tccl_timeout_flag_create) that is set to 1 when a wait expires */
@@ -256,6 +257,8 @@ typedef struct {
 } tccl_pipeline_cfg;
 
 #define TCCL_PIPE_DRAW_PLACES 1 /* workgroups draw their places when they start (see above) */
+#define TCCL_PIPE_OWN_BARRIERS 2 /* tccl_two_shot_all_reduce_rank only: the kernel begins and ends with the
+                                    blockwise barrier itself (see there) */
 
 size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int dtype, size_t chunk_elems);
 int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs,
@@ -304,7 +307,12 @@ int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *
  * every rank, the W launches running at the same time, tccl_blockwise_barrier() before and
  * after).  The barrier between the two shots is then exactly the reference's construct: a
  * blockwise barrier between kernels of different owners (triton_barrier.py:39-142), inside the
- * kernel.  `out` = this rank's output or NULL (the result is in bufs[rank] either way). */
+ * kernel.  `out` = this rank's output or NULL (the result is in bufs[rank] either way).
+ * With TCCL_PIPE_OWN_BARRIERS in cfg->flags the kernel also begins and ends with that barrier, as
+ * the reference's kernels begin with it (triton_one_shot_all_reduce_no_128.py:46), and no
+ * tccl_blockwise_barrier() before or after is needed: one launch per rank per collective.  The pads
+ * then hold three rows of slots per workgroup, pad_bytes >= 4 * (3 * world + TCCL_PAD_CONTROL_WORDS).
+ * An empty input launches nothing and orders nothing. */
 int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void *const *signal_pads,
                                   size_t pad_bytes, int world, int rank, size_t numel, int dtype,
                                   const tccl_pipeline_cfg *cfg, void *stream);

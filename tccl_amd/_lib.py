@@ -29,6 +29,7 @@ CFG_STREAMING = 16
 CFG_PHASED = 32
 
 PIPE_DRAW_PLACES = 1
+PIPE_OWN_BARRIERS = 2
 
 
 class TcclError(RuntimeError):

@@ -216,7 +216,8 @@ def all_reduce(tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
     every size; the other two exist for what they model across GPUs."""
     if algorithm not in ("auto", "one_shot", "two_shot", "double_tree"):
         raise ValueError(f"unknown all-reduce algorithm {algorithm!r}")
-    owner = _owner_world(rendezvous(tensor).group, "all_reduce")
+    # (inside a per-rank thread program the group only forms at the collective's own rendezvous)
+    owner = _owner_world(rendezvous(tensor).group, "all_reduce") if spmd.current_rank() is None else None
     if owner is not None:              # ranks are processes: there the three really differ, by size
         return owner.all_reduce(tensor, algorithm)
     if algorithm in ("auto", "one_shot"):
@@ -302,7 +303,9 @@ def double_tree_all_reduce(tensor: torch.Tensor, *, chunk_elems: int = 0,
     when ``fused`` is None too, where it is the fastest of the three."""
     dtype = _sum_dtype(tensor)
     assert tensor.numel() % _vec_elems(tensor) == 0, "The number of elements must be 128-bit aligned."
-    owner = _owner_world(rendezvous(tensor).group, "double_tree_all_reduce", needed=True)
+    owner = None
+    if spmd.current_rank() is None:    # (a per-rank thread program's group only forms at the collective's own rendezvous)
+        owner = _owner_world(rendezvous(tensor).group, "double_tree_all_reduce", needed=True)
     if owner is not None:
         # ranks are processes: this rank's own launch of the pipelined kernel between barriers; running
         # the node steps of all ranks from here would reduce the mapped buffers W times over

@@ -10,8 +10,8 @@
 //  * one slot per (chunk, sender) instead of one per (block, sender), so a sender never has
 //    to wait for the receiver to drain the previous chunk's signal (the reference's send
 //    spins on a compare-and-swap 0 -> 1 for that); every slot has exactly one writer and
-//    one reader per call, so plain release stores and acquire loads replace the
-//    compare-and-swap loops;
+//    one reader per call, so a plain store raises a flag (the wait is still the reference's
+//    compare-and-swap 1 -> 0);
 //  * the reader writes the slot back to 0 after it has seen the signal, so a pad that starts
 //    zero-filled is zero-filled again after every completed call (the property that makes the
 //    reference's barrier usable under graph replay);
@@ -211,6 +211,35 @@ __device__ __forceinline__ void report_timeout(uint32_t *ctl, uint32_t *report)
     if (report != nullptr) __hip_atomic_store(report, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// Take a raised flag: polls the slot with a compare-and-swap 1 -> 0, the reference's own wait
+// (triton_barrier.py:108-118), until it succeeds or the wait's budget is used up.  A device-scope
+// read-modify-write is carried out where all XCDs meet, so the poll sees the flag wherever its
+// sender ran, and seeing and lowering it are one step.
+//
+// The polls back off.  A launch that begins with a barrier may have a thousand workgroups
+// waiting for a rank that is still busy with the kernel before its collective, and every poll
+// goes to the few memory channels that hold the pads -- channels which that rank's kernel needs
+// as well.  So the first 64 polls come about 0.2 us apart, and the pause doubles with every
+// further 64 polls up to about 30 us: a flag is still taken within a fraction of the time it
+// has been waited for.  The budget counts pauses, not polls: spin_limit units of about 0.2 us.
+__device__ __forceinline__ bool take_flag(uint32_t *slot, uint32_t spin_limit, uint32_t *spent)
+{
+    uint32_t nap = 1, round = 0;
+    for (;;) {
+        uint32_t expect = 1u;
+        if (__hip_atomic_compare_exchange_strong(slot, &expect, 0u, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT))
+            return true;
+        *spent += nap;
+        if (*spent >= spin_limit) return false;
+        for (uint32_t i = 0; i < nap; ++i) __builtin_amdgcn_s_sleep(8);
+        if (++round == 64) {
+            round = 0;
+            if (nap < 128) nap *= 2;
+        }
+    }
+}
+
 // Coherence between workgroups on different XCDs (each XCD has its own L2) without flushing
 // or invalidating whole caches: every store of this kernel is a device-scope store (sc1: it
 // is written through to memory and acknowledged from there) and every load of data that a
@@ -227,8 +256,8 @@ __device__ __forceinline__ void send_signals(uint32_t *slot0, uint32_t *slot1)
     }
 }
 
-// Wait until every non-null slot has been raised, and lower it again.  One lane polls (a
-// device-scope load); the result reaches the other lanes through LDS, and the barrier keeps
+// Wait until every non-null slot has been raised, and lower it again.  One lane polls (with
+// take_flag); the result reaches the other lanes through LDS, and the barrier keeps
 // every lane's later loads behind the poll that saw the flag.  Returns false after
 // spin_limit polls without success (counted in the control words); the caller then leaves the
 // kernel.
@@ -244,14 +273,7 @@ __device__ __forceinline__ bool wait_signals(uint32_t *slot0, uint32_t *slot1, u
         for (int i = 0; i < 2; ++i) {
             uint32_t *s = slots[i];
             if (s == nullptr || !ok) continue;
-            while (__hip_atomic_load(s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
-                if (++polls >= spin_limit) {
-                    ok = false;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-            if (ok) __hip_atomic_store(s, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ok = take_flag(s, spin_limit, &polls);
         }
         if (!ok) report_timeout(ctl, report);
         *lds_ok = ok ? 1 : 0;
@@ -487,12 +509,26 @@ static size_t workgroups_per_rank(size_t units, size_t most, int world, bool tie
 // With the registers the signalling kernels need that is 2 to 5 per unit.  Never more than 6:
 // a signalling grid of 8 per unit once timed out for a reason that was never established, so
 // that shape stays unreachable whatever a kernel's register use becomes.
+//
+// waits_at_entry: the kernel's workgroups wait for their peers before they do anything (a
+// leading barrier), and the peers' launches may arrive much later, behind other kernels.  Then
+// the occupancy the runtime reports cannot be relied on: a wave's registers are one contiguous
+// block of its SIMD's 512, short-lived waves of other kernels that come and go between the
+// arrivals leave the waiting waves scattered over the file, and the holes between them may each
+// be too small for the late launch's waves although their sum is not.  (Measured with 8
+// processes at the reported 4 per unit: the last rank's launch got 2 of its 128 workgroups
+// placed and the other 896 waited for it until their waits expired.)  With n waves of v
+// registers per SIMD wanted, n - 1 badly placed ones leave a hole of at least
+// (512 - (n - 1) v) / n, which holds the n-th for n <= (512 + v) / (2 v): half the reported
+// figure, rounded up.  Only as many workgroups as that are launched, so the last arrival
+// always finds room.
 template <class K>
-static int resident_for(K kernel)
+static int resident_for(K kernel, bool waits_at_entry = false)
 {
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kPhasedBlock, 0) != hipSuccess || per_cu < 1) return 0;
     if (per_cu > kMaxSignallingPerUnit) per_cu = kMaxSignallingPerUnit;
+    if (waits_at_entry) per_cu = (per_cu + 1) / 2;
     return per_cu * compute_units();
 }
 
@@ -696,6 +732,7 @@ struct TwoShotArgs {
     int world, wgs_per_rank;
     int draw;         // 1 = workgroups draw their places when they start, 0 = places follow the hardware index
     int only_rank;    // >= 0: the launch holds this rank's workgroups only (one launch per rank); -1: all ranks'
+    int own_barriers; // one launch per rank: the kernel also begins and ends with the blockwise barrier
     uint32_t *ctl;    // control words at the end of pad 0 (place counters ... time-outs)
     uint32_t *report; // optional host word set to 1 when a wait expires
 };
@@ -703,33 +740,26 @@ struct TwoShotArgs {
 // The reference's blockwise barrier (triton_barrier.py:39-142) between the workgroups with
 // the same index g of all W virtual ranks: lane i < W of the first wave raises slot
 // `g * W + rank` in rank i's pad and waits for slot `g * W + i` in the own pad, which it
-// lowers again (each slot has one writer and one reader, so the reference's compare-and-swap
-// loops become a store and a polling load).  Everything the workgroup stored before the
+// lowers again (each slot has one writer and one reader, so the sender's compare-and-swap 0 -> 1
+// of the reference becomes a plain store; the wait is the reference's compare-and-swap 1 -> 0,
+// take_flag).  Everything the workgroup stored before the
 // barrier is visible to its peers' device-scope loads after it.  Returns false when a wait
 // expired (counted in the control words).
-__device__ __forceinline__ bool blockwise_barrier(const TwoShotArgs &a, int rank, uint32_t g, int *lds_ok)
+__device__ __forceinline__ bool blockwise_barrier(const TwoShotArgs &a, int rank, uint32_t row, int *lds_ok)
 {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     const int lane = threadIdx.x;
     if (lane < a.world && lane != rank) {
-        const uint32_t base = g * static_cast<uint32_t>(a.world);
+        const uint32_t base = row * static_cast<uint32_t>(a.world);
         __hip_atomic_store(a.pad[lane] + base + rank, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         uint32_t *mine = a.pad[rank] + base + lane;
         uint32_t polls = 0;
-        bool ok = true;
-        while (__hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
-            if (++polls >= a.spin_limit) {
-                ok = false;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-        }
-        if (ok)
-            __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else
+        const bool ok = take_flag(mine, a.spin_limit, &polls);
+        if (!ok) {
             report_timeout(a.ctl, a.report);
-        if (!ok) *lds_ok = 0; // any lane that failed clears the flag
+            *lds_ok = 0; // any lane that failed clears the flag
+        }
     }
     __syncthreads();
     return *lds_ok != 0;
@@ -748,10 +778,18 @@ __device__ __forceinline__ bool blockwise_barrier(const TwoShotArgs &a, int rank
 // inputs, whose shares it spreads over many more workgroups.
 constexpr int kTwoShotVecs = 4;
 
-template <class Sum, int W>
+//
+// PEERS_MAY_STILL_WRITE (one launch per rank): the kernel may have started before a peer's
+// producer kernel ended, so shot 1 reads with device-scope loads too; and with a.own_barriers
+// the kernel begins with the barrier that says "every rank's input is in place" (row G + g of
+// the pads) and ends with the one that says "every rank has read what it needs from every
+// buffer" (row 2 G + g) -- three barriers in a row on three different rows, so a flag is never
+// raised over one that its reader has not consumed, within a call and from call to call.
+template <class Sum, int W, bool PEERS_MAY_STILL_WRITE>
 __device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, uint32_t g, int &lds_ok)
 {
     constexpr int VECS = kTwoShotVecs;
+    constexpr int LAUX = PEERS_MAY_STILL_WRITE ? kAuxLoadDevice : kAuxLoadStream;
     constexpr int U = PhasedUnroll<W>::value < VECS ? PhasedUnroll<W>::value : VECS;
     constexpr int KMAX = VECS / U;
     constexpr uint32_t span = kPhasedBlock * U * kVecBytes;
@@ -759,6 +797,8 @@ __device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, ui
     const uint32_t G = a.wgs_per_rank;
     if (threadIdx.x == 0) lds_ok = 1;
     // (the barrier's first __syncthreads orders this store before any lane's clear)
+    const bool own_barriers = PEERS_MAY_STILL_WRITE && W > 1 && a.own_barriers != 0;
+    if (own_barriers && !blockwise_barrier(a, rank, G + g, &lds_ok)) return;
 
     const char *src[W];
 #pragma unroll
@@ -773,15 +813,15 @@ __device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, ui
         if (a.out[rank] != nullptr) {
             char *const dst[2] = {a.buf[rank], a.out[rank]};
             if (full)
-                sum_tile_phased<Sum, W, 2, U, KMAX, true, Sum::kPaceLoads>(csrc, dst, share_off + t, valid, KMAX);
+                sum_tile_phased<Sum, W, 2, U, KMAX, true, Sum::kPaceLoads, LAUX>(csrc, dst, share_off + t, valid, KMAX);
             else
-                sum_tile_phased<Sum, W, 2, U, KMAX, false, Sum::kPaceLoads>(csrc, dst, share_off + t, valid, kcount);
+                sum_tile_phased<Sum, W, 2, U, KMAX, false, Sum::kPaceLoads, LAUX>(csrc, dst, share_off + t, valid, kcount);
         } else {
             char *const dst[1] = {a.buf[rank]};
             if (full)
-                sum_tile_phased<Sum, W, 1, U, KMAX, true, Sum::kPaceLoads>(csrc, dst, share_off + t, valid, KMAX);
+                sum_tile_phased<Sum, W, 1, U, KMAX, true, Sum::kPaceLoads, LAUX>(csrc, dst, share_off + t, valid, KMAX);
             else
-                sum_tile_phased<Sum, W, 1, U, KMAX, false, Sum::kPaceLoads>(csrc, dst, share_off + t, valid, kcount);
+                sum_tile_phased<Sum, W, 1, U, KMAX, false, Sum::kPaceLoads, LAUX>(csrc, dst, share_off + t, valid, kcount);
         }
     }
     if (W == 1) return;
@@ -805,6 +845,7 @@ __device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, ui
             }
         }
     }
+    if (own_barriers) (void)blockwise_barrier(a, rank, 2 * G + g, &lds_ok);
 }
 
 template <class Sum, int W>
@@ -814,15 +855,17 @@ __global__ void __launch_bounds__(kPhasedBlock) two_shot_kernel(TwoShotArgs a)
     __shared__ uint32_t lds_place[2];
     int rank;
     uint32_t g;
-    if (a.only_rank >= 0) {
-        // one launch per rank: the barrier between the shots is then the reference's own
-        // construct, a barrier between the kernels of different owners
-        rank = a.only_rank;
-        g = blockIdx.x;
-    } else {
-        take_place(a.ctl, a.draw != 0, W, a.wgs_per_rank, &rank, &g, lds_place);
-    }
-    if (g != kNoPlace) two_shot_body<Sum, W>(a, rank, g, lds_ok);
+    take_place(a.ctl, a.draw != 0, W, a.wgs_per_rank, &rank, &g, lds_place);
+    if (g != kNoPlace) two_shot_body<Sum, W, false>(a, rank, g, lds_ok);
+}
+
+// One launch per rank: the barrier between the shots is then the reference's own construct, a
+// barrier between the kernels of different owners.
+template <class Sum, int W>
+__global__ void __launch_bounds__(kPhasedBlock) two_shot_rank_kernel(TwoShotArgs a)
+{
+    __shared__ int lds_ok;
+    two_shot_body<Sum, W, true>(a, a.only_rank, blockIdx.x, lds_ok);
 }
 
 // What the entry point without caller-owned pads asks for before its kernel: zero the first
@@ -851,13 +894,19 @@ template <class Sum, int W>
 static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, const ClearRequest *clear, hipStream_t s)
 {
     static std::once_flag once;
-    static int resident = 0;
-    std::call_once(once, [] { resident = resident_for(two_shot_kernel<Sum, W>); });
+    static int resident_one = 0, resident_rank = 0, resident_rank_entry = 0;
+    std::call_once(once, [] {
+        resident_one = resident_for(two_shot_kernel<Sum, W>);
+        resident_rank = resident_for(two_shot_rank_kernel<Sum, W>);
+        resident_rank_entry = resident_for(two_shot_rank_kernel<Sum, W>, true);
+    });
+    const int resident = a.only_rank < 0 ? resident_one : (a.own_barriers ? resident_rank_entry : resident_rank);
     if (resident < W) return hip_code(hipErrorLaunchOutOfResources);
     constexpr size_t tile_bytes = static_cast<size_t>(kPhasedBlock) * kTwoShotVecs * kVecBytes;
     const size_t tiles = (a.share_bytes + tile_bytes - 1) / tile_bytes;
-    // one slot per (workgroup index, sender) in every pad; the last words of pad 0 are the control words
-    const size_t fit = (pad_words - kCtlWords) / W;
+    // one slot per (workgroup index, sender) in every pad -- three with the kernel's own leading and
+    // trailing barriers; the last words of pad 0 are the control words
+    const size_t fit = (pad_words - kCtlWords) / (static_cast<size_t>(W) * (a.own_barriers ? 3 : 1));
     if (fit < 1) return TCCL_EINVAL;
     size_t per_rank;
     if (wgs_wanted > 0) {
@@ -878,9 +927,10 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, cons
         const hipError_t ce = hipGetLastError();
         if (ce != hipSuccess) return hip_code(ce);
     }
-    const size_t ranks_in_launch = a.only_rank >= 0 ? 1 : W;
-    hipLaunchKernelGGL((two_shot_kernel<Sum, W>), dim3(static_cast<unsigned>(per_rank * ranks_in_launch)),
-                       dim3(kPhasedBlock), 0, s, a);
+    if (a.only_rank >= 0)
+        hipLaunchKernelGGL((two_shot_rank_kernel<Sum, W>), dim3(static_cast<unsigned>(per_rank)), dim3(kPhasedBlock), 0, s, a);
+    else
+        hipLaunchKernelGGL((two_shot_kernel<Sum, W>), dim3(static_cast<unsigned>(per_rank * W)), dim3(kPhasedBlock), 0, s, a);
     const hipError_t e = hipGetLastError();
     if (e == hipSuccess) guard.launched();
     return hip_code(e);
@@ -938,6 +988,7 @@ static int two_shot_launch(void *const *bufs, void *const *outs, uint32_t *const
     a.ctl = a.pad[0] + pad_words - kCtlWords;
     a.report = cfg ? cfg->timeout_flag : nullptr;
     a.only_rank = only_rank;
+    a.own_barriers = (only_rank >= 0 && cfg && (cfg->flags & TCCL_PIPE_OWN_BARRIERS)) ? 1 : 0;
     a.draw = (only_rank < 0 && cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
     const int wgs = cfg ? cfg->workgroups : 0;
     return dtype == TCCL_BF16 ? launch_two_shot_world<Bf16Sum>(a, wgs, pad_words, clear, s)
@@ -973,7 +1024,8 @@ extern "C" int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void 
 {
     if (signal_pads == nullptr || world < 1 || world > TCCL_MAX_WORLD || rank < 0 || rank >= world) return TCCL_EINVAL;
     if (cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) return TCCL_EINVAL; // places are fixed by the rank's own launch
-    if (pad_bytes % 16 != 0 || pad_bytes < (static_cast<size_t>(world) + kCtlWords) * sizeof(uint32_t))
+    const size_t rows = (cfg && (cfg->flags & TCCL_PIPE_OWN_BARRIERS)) ? 3 : 1;
+    if (pad_bytes % 16 != 0 || pad_bytes < (rows * static_cast<size_t>(world) + kCtlWords) * sizeof(uint32_t))
         return TCCL_EINVAL;
     void *outs[TCCL_MAX_WORLD] = {};
     outs[rank] = out;
@@ -1030,17 +1082,8 @@ __device__ __forceinline__ bool rank_barrier(const RankArgs &a, uint32_t row, in
         __hip_atomic_store(a.pad[lane] + base + a.rank, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         uint32_t *mine = a.pad[a.rank] + base + lane;
         uint32_t polls = 0;
-        bool ok = true;
-        while (__hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
-            if (++polls >= a.spin_limit) {
-                ok = false;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-        }
-        if (ok)
-            __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else
+        const bool ok = take_flag(mine, a.spin_limit, &polls);
+        if (!ok)
             report_timeout(a.ctl, a.report);
         if (!ok) *lds_ok = 0;
     }
@@ -1140,7 +1183,7 @@ static int launch_sum_rank_w(const RankArgs &a, size_t tiles, int wgs, size_t pa
     // asked once per kernel: the answer depends on the kernel's register use only
     static std::once_flag once;
     static int resident = 0;
-    std::call_once(once, [] { resident = resident_for(sum_rank_kernel<Sum, W>); });
+    std::call_once(once, [] { resident = resident_for(sum_rank_kernel<Sum, W>, true); });
     return launch_rank_kernel(sum_rank_kernel<Sum, W>, resident, a, tiles, wgs, pad_words, s);
 }
 
@@ -1241,7 +1284,7 @@ extern "C" int tccl_all_gather_rank(void *const *bufs, void *out, void *const *s
     if (tiles < 1) tiles = 1;
     static std::once_flag once;
     static int resident = 0;
-    std::call_once(once, [] { resident = resident_for(gather_rank_kernel); });
+    std::call_once(once, [] { resident = resident_for(gather_rank_kernel, true); });
     return launch_rank_kernel(gather_rank_kernel, resident, a, tiles, cfg ? cfg->workgroups : 0,
                               pad_bytes / sizeof(uint32_t), static_cast<hipStream_t>(stream));
 }

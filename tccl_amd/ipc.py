@@ -152,7 +152,7 @@ class IpcWorld:
         rank's own at index ``rank``), as tensors over the mapped memory: what the reference gets
         from ``symm_mem.get_buffer(rank, ...)``.  Reading a peer's buffer is ordered against the
         peer's writes by ``barrier()`` like everything else."""
-        ptrs, nbytes, dtype = self._tables[tensor.data_ptr()]
+        ptrs, nbytes, dtype = self._tables[self._base(tensor)]
         return [_as_tensor(p, nbytes, self.device).view(dtype) for p in ptrs]
 
     def host_barrier(self) -> None:
@@ -189,21 +189,26 @@ class IpcWorld:
             self._tree_pads[nbytes] = _lib.ptr_array(self._exchange(self._alloc(nbytes), "kpad"))
         return self._tree_pads[nbytes]
 
-    def _own_launch(self, name: str, tensor: torch.Tensor, pad_bytes: int, tail_args, cfg) -> torch.Tensor:
-        ptrs, _, dtype = self._tables[tensor.data_ptr()]
+    def _own_launch(self, name: str, tensor: torch.Tensor, pad_bytes: int, tail_args, cfg,
+                    own_barriers: bool = False) -> torch.Tensor:
+        ptrs, _, dtype = self._tables[self._base(tensor)]
         code = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype]
         pads = self._kernel_pads(pad_bytes)
         use = _lib.PipelineCfg()
         if cfg is not None:
             ctypes.memmove(ctypes.byref(use), ctypes.byref(cfg), ctypes.sizeof(use))
         use.timeout_flag = self._flag
+        if own_barriers:
+            use.flags |= _lib.PIPE_OWN_BARRIERS            # the kernel begins and ends with the barrier itself
         out = torch.empty_like(tensor)
         stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
-        self.barrier()                                     # every rank's input is in place
+        if not own_barriers:
+            self.barrier()                                 # every rank's input is in place
         rc = getattr(self.lib, name)(_lib.ptr_array(ptrs), out.data_ptr(), pads, pad_bytes, self.world_size, self.rank,
                                      tensor.numel(), code, *tail_args, ctypes.byref(use), stream)
         _lib.check(name, rc)
-        self.barrier()                                     # every rank is done with buffers and pads
+        if not own_barriers:
+            self.barrier()                                 # every rank is done with buffers and pads
         return out
 
     def double_tree_all_reduce(self, tensor: torch.Tensor, chunk_elems: int = 0,
@@ -213,20 +218,25 @@ class IpcWorld:
         wait/send on signal pads in each other's memory, between a leading and a trailing barrier.
         Collective; the symmetric buffers are overwritten (every rank's ends up holding the sum,
         which is also returned).  Worlds of 2, 4 and 8."""
-        _, _, dtype = self._tables[tensor.data_ptr()]
+        _, _, dtype = self._tables[self._base(tensor)]
         code = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype]
         need = self.lib.tccl_double_tree_signal_pad_bytes(self.world_size, tensor.numel(), code, chunk_elems)
         if need == 0:
             raise ValueError("the pipelined double tree takes worlds of 2, 4 or 8 and whole 16-byte vectors")
         return self._own_launch("tccl_double_tree_all_reduce_pipelined_rank", tensor, need, (chunk_elems,), cfg)
 
-    def two_shot_all_reduce(self, tensor: torch.Tensor, cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+    def two_shot_all_reduce(self, tensor: torch.Tensor, cfg: Optional[_lib.PipelineCfg] = None,
+                            own_barriers: bool = True) -> torch.Tensor:
         """Two-shot all-reduce, this rank's own launch: reduce the own share from all buffers, meet
         the other ranks' kernels in the reference's blockwise barrier (triton_barrier.py:39-142,
         inside the kernel, as the reference uses it), gather the other shares.  Collective, in
         place (every buffer ends up holding the sum, which is also returned); bit-identical to
-        ``one_shot_all_reduce``.  The element count must be a multiple of W vectors."""
-        return self._own_launch("tccl_two_shot_all_reduce_rank", tensor, self.TWO_SHOT_PAD_BYTES, (), cfg)
+        ``one_shot_all_reduce``.  The element count must be a multiple of W vectors.
+        ``own_barriers``: the kernel also begins and ends with that barrier (one launch per rank);
+        False = a barrier launch before and after instead."""
+        if tensor.numel() == 0:
+            return torch.empty_like(tensor)
+        return self._own_launch("tccl_two_shot_all_reduce_rank", tensor, self.TWO_SHOT_PAD_BYTES, (), cfg, own_barriers)
 
     # Signal pad size of the one-shot kernels: two rows of slots for up to 512 workgroups per rank.
     ONE_SHOT_PAD_BYTES = 4 * (2 * 8 * 512 + 288)
