@@ -187,7 +187,6 @@ def two_shot_all_reduce(tensor: torch.Tensor) -> torch.Tensor:
     direction over the links instead of (W-1) whole buffers."""
     dtype = _sum_dtype(tensor)
     lib = _lib.load()
-    stream = _stream(tensor.device)
     with spmd.collective():
         symm = rendezvous(tensor)
         symm.group.check_signals()
@@ -196,6 +195,7 @@ def two_shot_all_reduce(tensor: torch.Tensor) -> torch.Tensor:
         owner = _owner_world(symm.group, "two_shot_all_reduce", needed=True)
         if owner is not None:          # in place there: every buffer ends up holding the result
             return owner.two_shot_all_reduce(tensor)
+        stream = _stream(tensor.device)
         per_rank = tensor.numel() // world
         shares = torch.empty((world, per_rank), dtype=tensor.dtype, device=tensor.device)
         output = torch.empty_like(tensor)

@@ -1352,7 +1352,8 @@ extern "C" int tccl_two_shot_all_reduce_static(void *const *bufs, void *const *o
     ClearRequest clear;
     clear.base = reinterpret_cast<uint32_t *>(base);
     clear.pad_words = static_cast<uint32_t>(kStaticPadBytes / sizeof(uint32_t));
-    clear.flag_words = static_cast<uint32_t>(TCCL_STATIC_MAX_WORKGROUPS) * world;
+    // every flag word a launch on these pads can touch, whatever count of workgroups it settles on
+    clear.flag_words = clear.pad_words - kCtlWords;
     clear.pads = world;
     return two_shot_launch(bufs, outs, pads, kStaticPadBytes, world, numel, dtype, cfg, &clear,
                            static_cast<hipStream_t>(stream));

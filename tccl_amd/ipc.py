@@ -45,6 +45,23 @@ def _as_tensor(ptr: int, nbytes: int, device) -> torch.Tensor:
     return torch.as_tensor(_DeviceBlock(ptr, nbytes), device=device)
 
 
+def _refuse_used_directory(directory: str, rank: int) -> None:
+    """The handle files have fixed names (``pad0.rank3``, ``buf1.rank0`` ...): in a directory that an
+    earlier run has used, this run's ranks would read that run's 64-byte handles and try to map
+    allocations that no longer exist.  A rank therefore refuses a directory that already holds a file
+    of its own rank (every rank writes before it reads, so in a fresh directory none can exist yet)."""
+    suffix = f".rank{rank}"
+    try:
+        names = os.listdir(directory)
+    except OSError as e:
+        raise RuntimeError(f"the rendezvous directory {directory!r} cannot be read: {e}") from None
+    old = sorted(n for n in names if n.endswith(suffix) or n.endswith(f".tmp{rank}"))
+    if old:
+        raise RuntimeError(f"the rendezvous directory {directory!r} already holds files of rank {rank} from another run "
+                           f"({', '.join(old[:3])}{' ...' if len(old) > 3 else ''}): every run needs a fresh directory "
+                           "(python -m tccl_amd.launch makes one)")
+
+
 class IpcWorld:
     """This process's view of W processes sharing one GPU.  ``directory`` is where the ranks leave
     their handles for each other (any place all of them can read and write)."""
@@ -56,6 +73,7 @@ class IpcWorld:
         if not (1 <= world_size <= _lib.MAX_WORLD and 0 <= rank < world_size):
             raise ValueError("rank/world_size out of range")
         self.rank, self.world_size, self.directory, self.timeout_s = rank, world_size, directory, timeout_s
+        _refuse_used_directory(directory, rank)
         self.device = torch.device(device)
         self.lib = _lib.load()
         self._allocs: List[int] = []          # own allocations
@@ -241,9 +259,35 @@ class IpcWorld:
     # Signal pad size of the one-shot kernels: two rows of slots for up to 512 workgroups per rank.
     ONE_SHOT_PAD_BYTES = 4 * (2 * 8 * 512 + 288)
 
+    # A one-shot collective is ONE launch with the barriers inside while its kernel moves at most this many
+    # bytes, and barrier launch + the library's full-size kernel + barrier launch above: a rank's own launch
+    # holds only 1/W of the workgroups that are certain to find room beside the peers' launches and works in
+    # 16 KiB tiles, which costs more than two extra launches once the data is large (8 processes on one
+    # MI355X, all-reduce of 8 x 16 MiB = 144 MiB moved: 298-313 us fused against 287-328 us; 8 x 64 MiB:
+    # 1,110 against 880-900 us; reduce-scatter of 8 x 256 MiB = 288 MiB moved: 560 against 460-500 us, of
+    # 8 x 64 MiB = 72 MiB: 172-183 against 199-233 us; profiles/ipc_forms_one_gpu_8_4_2_processes.txt).
+    FUSED_MAX_MOVED_BYTES = 128 << 20
+
     def _one_shot(self, name: str, tensor: torch.Tensor, out: torch.Tensor, size_arg: int, with_dtype: bool,
-                  cfg: Optional[_lib.PipelineCfg]) -> torch.Tensor:
+                  cfg: Optional[_lib.PipelineCfg], moved_bytes: int = 0, fused: Optional[bool] = None) -> torch.Tensor:
         ptrs, _, dtype = self._tables[self._base(tensor)]
+        if fused is None:
+            fused = moved_bytes <= self.FUSED_MAX_MOVED_BYTES
+        if not fused:
+            if cfg is not None:
+                raise ValueError("a PipelineCfg applies to the one-launch form only (fused=True)")
+            stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+            plain = name[:-len("_rank")]
+            args = [_lib.ptr_array(ptrs), self.world_size]
+            if plain == "tccl_reduce_scatter_sum":
+                args.append(self.rank)
+            args += [out.data_ptr(), size_arg]
+            if with_dtype:
+                args.append({torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype])
+            self.barrier()                                     # every rank's input is in place
+            _lib.check(plain, getattr(self.lib, plain)(*args, stream))
+            self.barrier()                                     # every rank has read every buffer
+            return out
         pads = self._kernel_pads(self.ONE_SHOT_PAD_BYTES)
         use = _lib.PipelineCfg()
         if cfg is not None:
@@ -266,18 +310,21 @@ class IpcWorld:
         return base
 
     def one_shot_all_reduce(self, tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
-                            cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+                            cfg: Optional[_lib.PipelineCfg] = None, fused: Optional[bool] = None) -> torch.Tensor:
         """``one_shot_all_reduce`` the way the reference's kernel runs it (triton_one_shot_all_reduce_no_128.py:35-64):
         this rank's ONE launch, which meets the peers' launches in ``blockwise_barrier`` first (:46), sums all
         W buffers in rank order into a fresh output, and meets the peers again before it ends (so the buffers
-        may be refilled as soon as the call's kernel is done).  Collective: every rank calls it."""
+        may be refilled as soon as the call's kernel is done).  Collective: every rank calls it.
+        ``fused``: None = that form up to ``FUSED_MAX_MOVED_BYTES``, above it a barrier launch, the
+        library's full-size kernel and a barrier launch (same values, same guarantees); True / False force one."""
         assert tensor.dtype in (torch.bfloat16, torch.float32), "Only bfloat16 (and float32) is supported for now."
         assert tensor.numel() % (16 // tensor.element_size()) == 0, "The number of elements must be 128-bit aligned."
         output = torch.empty_like(tensor) if out is None else out
-        return self._one_shot("tccl_all_reduce_sum_rank", tensor, output, tensor.numel(), True, cfg)
+        moved = (self.world_size + 1) * tensor.numel() * tensor.element_size()
+        return self._one_shot("tccl_all_reduce_sum_rank", tensor, output, tensor.numel(), True, cfg, moved, fused)
 
     def reduce_scatter(self, tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
-                       cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+                       cfg: Optional[_lib.PipelineCfg] = None, fused: Optional[bool] = None) -> torch.Tensor:
         """``one_shot_reduce_scatter`` as one launch of this rank with the barriers inside the kernel
         (triton_reduce_scatter.py:59-92; the reference has its leading barrier commented out, :70)."""
         assert tensor.dtype in (torch.bfloat16, torch.float32), "Only bfloat16 (and float32) is supported for now."
@@ -285,34 +332,47 @@ class IpcWorld:
             "The number of elements must be 128-bit aligned."
         per_rank = tensor.numel() // self.world_size
         output = torch.empty((per_rank,), dtype=tensor.dtype, device=tensor.device) if out is None else out
-        return self._one_shot("tccl_reduce_scatter_sum_rank", tensor, output, tensor.numel(), True, cfg)
+        moved = (self.world_size + 1) * per_rank * tensor.element_size()
+        return self._one_shot("tccl_reduce_scatter_sum_rank", tensor, output, tensor.numel(), True, cfg, moved, fused)
 
     def all_gather(self, tensor: torch.Tensor, *, out: Optional[torch.Tensor] = None,
-                   cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+                   cfg: Optional[_lib.PipelineCfg] = None, fused: Optional[bool] = None) -> torch.Tensor:
         """``one_shot_all_gather`` as one launch of this rank with the barriers inside the kernel
         (triton_all_gather.py:32-63, leading barrier :43)."""
         nbytes = tensor.numel() * tensor.element_size()
         assert nbytes % 16 == 0, "The number of elements must be 128-bit aligned."
         if out is None:
             out = torch.empty((self.world_size, *tensor.shape), dtype=tensor.dtype, device=tensor.device)
-        return self._one_shot("tccl_all_gather_rank", tensor, out, nbytes, False, cfg)
+        return self._one_shot("tccl_all_gather_rank", tensor, out, nbytes, False, cfg, 2 * self.world_size * nbytes, fused)
 
-    # All-reduce by size, measured with 8 processes on one MI355X (python -m tccl_amd.launch
-    # --nproc-per-node 8 benchlib/ipc_forms.py, us per collective, one-shot / two-shot / double tree):
-    # see ONE_SHOT_MAX_BYTES below.  Across GPUs the one-shot form moves (W-1) whole buffers per rank
-    # over the links and the thresholds would sit far lower; on one GPU they are what was measured.
-    ONE_SHOT_MAX_BYTES = 1 << 62
+    # all_reduce(algorithm="auto"): one-shot up to this many bytes per buffer, two-shot above it in worlds of more
+    # than 4.  Measured with 8 processes on one MI355X (python -m tccl_amd.launch --nproc-per-node 8
+    # benchlib/ipc_forms.py, us per collective, one-shot / two-shot / double tree; profiles/
+    # ipc_forms_one_gpu_8_4_2_processes.txt): 1 MiB 58-72 / 139-184 / 236-310; 4 MiB 105-118 / 162-203 / 267-341;
+    # 16 MiB 287-313 / 244-287 / 339-413; 64 MiB 880-900 / 700-730 / 850-925; 256 MiB 3,300 / 2,600-2,790 /
+    # 2,880-2,990.  With 4 processes (and with 2) the one-shot form is the fastest at every size: 64 MiB
+    # 264-269 / 311 / 386, 256 MiB 923 / 1,250 / 1,245; worlds of 5 to 7 were not measured and take the rule
+    # of 8.  The double tree is never the fastest on one GPU and is run by name only.  Across GPUs the
+    # one-shot form moves W - 1 whole buffers per rank over the links and the thresholds would sit far lower.
+    ONE_SHOT_MAX_BYTES = 8 << 20
+    TWO_SHOT_MIN_WORLD = 5
+
+    def auto_algorithm(self, tensor: torch.Tensor) -> str:
+        """What ``all_reduce(tensor, "auto")`` runs."""
+        nbytes = tensor.numel() * tensor.element_size()
+        vec = 16 // tensor.element_size()
+        if nbytes > self.ONE_SHOT_MAX_BYTES and self.world_size >= self.TWO_SHOT_MIN_WORLD \
+                and tensor.numel() % (vec * self.world_size) == 0:
+            return "two_shot"
+        return "one_shot"
 
     def all_reduce(self, tensor: torch.Tensor, algorithm: str = "auto") -> torch.Tensor:
         """All-reduce of this rank's buffer by the named algorithm -- ``"one_shot"`` (fresh output, buffers
         untouched), ``"two_shot"`` or ``"double_tree"`` (both in place: every buffer ends up holding the
-        result, which is also returned) -- or ``"auto"``: the fastest of the three for the buffer's size."""
+        result, which is also returned) -- or ``"auto"``: the fastest of the three for the buffer's size and the world's (``auto_algorithm``; note
+        that it may work in place)."""
         if algorithm == "auto":
-            nbytes = tensor.numel() * tensor.element_size()
-            vec = 16 // tensor.element_size()
-            algorithm = "one_shot"
-            if nbytes > self.ONE_SHOT_MAX_BYTES and tensor.numel() % (vec * self.world_size) == 0:
-                algorithm = "two_shot"
+            algorithm = self.auto_algorithm(tensor)
         if algorithm == "one_shot":
             return self.one_shot_all_reduce(tensor)
         if algorithm == "two_shot":

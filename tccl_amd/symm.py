@@ -103,7 +103,10 @@ class SymmGroup:
         for this group has expired since the last check: that collective left partial results
         in the buffers and its outputs.  Costs one read of host memory, no synchronisation, so
         every collective on the group calls it first; after a time-out it waits for the device,
-        zeroes the pads and the flag (the group is usable again) and raises."""
+        zeroes the pads and the flag (the group is usable again) and raises.  Because the flag is read
+        without waiting for the device, a time-out can surface one collective late: then the collective
+        launched just before the raise ran on pads that still held the expired one's flags, and its
+        results are suspect as well."""
         if self._timeout_flag is None or self._timeout_flag[0] == 0:
             return
         torch.cuda.synchronize(self.tensors[0].device)

@@ -34,6 +34,12 @@ ONE_SHOT_SHAPES = (("small", 8 * 5, torch.bfloat16), ("ragged", 8 * 4099, torch.
                    ("big", 8 * 131_072, torch.bfloat16))
 
 
+def AUTO_SIZES(world_size, edge):
+    """(name, bf16 elements): small; at the threshold of "auto"; one step (W vectors) above it; a buffer
+    large enough that a one-shot all-reduce is three launches again."""
+    return (("small", 8 * world_size * 33), ("at", edge), ("above", edge + 8 * world_size), ("large", 4 * edge))
+
+
 def fill(t, numel, dtype, seed):
     torch.manual_seed(seed)
     if dtype == torch.bfloat16:
@@ -166,6 +172,25 @@ def main():
             world.host_barrier()
         world.close()
         return 42 if reported else 1
+
+    if mode == "auto":
+        # IpcWorld.all_reduce: every algorithm by name and "auto" at one size either side of its threshold
+        # (and one size above the point where a one-shot collective stops being one launch)
+        edge = world.ONE_SHOT_MAX_BYTES // 2                     # bf16 elements at the threshold
+        for tag, numel in AUTO_SIZES(world_size, edge):
+            t = world.empty(numel, torch.bfloat16)
+            for algorithm in ("auto", "one_shot", "two_shot", "double_tree"):
+                fill(t, numel, torch.bfloat16, rank)              # the in-place forms overwrite the buffer
+                picked = world.auto_algorithm(t) if algorithm == "auto" else algorithm
+                via_wrapper = algorithm in ("auto", "two_shot")   # the reference-side names lead to the same place
+                out = tccl_amd.all_reduce(t, algorithm) if via_wrapper else world.all_reduce(t, algorithm)
+                world.check()
+                save(directory, f"auto_{tag}.{algorithm}", rank, out)
+                if rank == 0:
+                    print(f"PICKED {tag} {algorithm} {picked}", flush=True)
+                world.host_barrier()                              # nobody refills before everybody has saved
+        world.close()
+        return 0
 
     if mode == "reference_mains":
         # the self-tests at the bottom of the reference's four kernel files, with a process per rank

@@ -108,3 +108,107 @@ def test_world_from_environment_needs_a_launcher(monkeypatch):
         monkeypatch.delenv(name, raising=False)
     with pytest.raises(RuntimeError, match="tccl_amd.launch"):
         ipc.IpcWorld.from_env()
+
+
+def test_a_rank_of_a_process_group_never_runs_its_peers_work():
+    """A buffer whose peers belong to other processes: everything that would launch every rank's steps
+    from this process refuses it (W processes doing that would reduce the mapped buffers W times over)."""
+    from tccl_amd import symm
+    own = torch.zeros(64, dtype=torch.bfloat16)
+    others = [torch.zeros(64, dtype=torch.bfloat16) for _ in range(3)]
+    ptrs = [others[0].data_ptr(), own.data_ptr(), others[1].data_ptr(), others[2].data_ptr()]
+    group = symm.register_remote(own, 1, ptrs)                       # no IpcWorld behind it
+    assert tccl_amd.rendezvous(own).rank == 1 and group.world is None
+    with pytest.raises(RuntimeError, match="other processes"):
+        tccl_amd.double_tree_all_reduce(own)
+    with pytest.raises(RuntimeError, match="other processes"):
+        tccl_amd.two_shot_all_reduce(own)
+    with pytest.raises(RuntimeError, match="other processes"):
+        tccl_amd.all_reduce(own, "double_tree")
+    with pytest.raises(RuntimeError, match="other processes"):
+        tccl_amd.double_tree_all_reduce_world(group)
+    with pytest.raises(RuntimeError, match="other processes"):
+        tccl_amd.two_shot_all_reduce_world(group)
+    with pytest.raises(RuntimeError, match="other processes"):
+        tccl_amd.DoubleTreePlan(group)
+    with pytest.raises(ValueError, match="unknown all-reduce algorithm"):
+        tccl_amd.all_reduce(own, "ring")
+    tccl_amd.unregister(group)
+
+
+def test_wrappers_hand_a_process_groups_collectives_to_its_world():
+    """With the IpcWorld behind the group the reference's names run that world's per-rank forms."""
+    from tccl_amd import symm
+
+    class World:
+        world_size = 2
+        calls = []
+
+        def one_shot_all_reduce(self, t, out=None):
+            self.calls.append("one_shot")
+            return out
+
+        def reduce_scatter(self, t, out=None):
+            self.calls.append("reduce_scatter")
+            return out
+
+        def all_gather(self, t, out=None):
+            self.calls.append("all_gather")
+            return out
+
+        def two_shot_all_reduce(self, t):
+            self.calls.append("two_shot")
+            return t
+
+        def double_tree_all_reduce(self, t, chunk_elems=0):
+            self.calls.append("double_tree")
+            return t
+
+        def all_reduce(self, t, algorithm):
+            self.calls.append("all_reduce:" + algorithm)
+            return t
+
+    own, other = torch.zeros(64, dtype=torch.bfloat16), torch.zeros(64, dtype=torch.bfloat16)
+    world = World()
+    group = symm.register_remote(own, 0, [own.data_ptr(), other.data_ptr()], world=world)
+    assert group.world is world
+    tccl_amd.one_shot_all_reduce(own)
+    tccl_amd.reduce_scatter(own)
+    tccl_amd.all_gather(own, 2)
+    tccl_amd.two_shot_all_reduce(own)
+    tccl_amd.double_tree_all_reduce(own)
+    tccl_amd.all_reduce(own, "auto")
+    assert world.calls == ["one_shot", "reduce_scatter", "all_gather", "two_shot", "double_tree", "all_reduce:auto"]
+    with pytest.raises(ValueError, match="per-rank"):
+        tccl_amd.one_shot_all_reduce(own, cfg=tccl_amd.LaunchCfg())
+    with pytest.raises(ValueError, match="per-rank pipelined kernel only"):
+        tccl_amd.double_tree_all_reduce(own, fused=True)
+    tccl_amd.unregister(group)
+
+
+def test_ipc_world_refuses_a_directory_another_run_has_used(tmp_path):
+    """The handle files have fixed names: a rank that found its own files from an earlier run would go on
+    to map allocations that no longer exist.  Refused before anything touches the GPU."""
+    from tccl_amd import ipc
+    (tmp_path / "pad0.rank1").write_bytes(b"x" * 64)
+    with pytest.raises(RuntimeError, match="another run"):
+        ipc.IpcWorld(1, 2, str(tmp_path))
+    ipc._refuse_used_directory(str(tmp_path), 0)                     # rank 0 has no file there yet: fine
+    with pytest.raises(RuntimeError, match="cannot be read"):
+        ipc.IpcWorld(0, 2, str(tmp_path / "missing"))
+
+
+def test_ipc_world_picks_the_all_reduce_by_size_and_world():
+    from tccl_amd import ipc
+
+    class Fake(ipc.IpcWorld):
+        def __init__(self, world_size):                               # no GPU, no files
+            self.world_size, self.rank = world_size, 0
+
+    mib = 1 << 19                                                     # bf16 elements per MiB
+    assert Fake(8).auto_algorithm(torch.empty(8 * mib, dtype=torch.bfloat16)) == "one_shot"
+    assert Fake(8).auto_algorithm(torch.empty(8 * mib + 64, dtype=torch.bfloat16)) == "two_shot"
+    assert Fake(8).auto_algorithm(torch.empty(8 * mib + 8, dtype=torch.bfloat16)) == "one_shot"      # shares would be ragged
+    assert Fake(4).auto_algorithm(torch.empty(64 * mib, dtype=torch.bfloat16)) == "one_shot"
+    assert Fake(2).auto_algorithm(torch.empty(64 * mib, dtype=torch.bfloat16)) == "one_shot"
+    assert Fake(5).auto_algorithm(torch.empty(5 * 16 * mib, dtype=torch.float32)) == "two_shot"

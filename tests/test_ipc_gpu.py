@@ -169,6 +169,29 @@ def test_reset_clears_the_pads_of_the_signalling_kernels(tmp_path):
             assert torch.equal(got, want), f"round {round_} rank {r}"
 
 
+def test_all_reduce_by_name_and_auto_either_side_of_the_threshold(tmp_path):
+    """IpcWorld.all_reduce with 8 processes: "auto" takes the one-shot kernel up to ONE_SHOT_MAX_BYTES per buffer
+    and the two-shot kernel one step above it; every algorithm by name at every size.  One-shot and two-shot
+    against the oracle's all-reduce, the double tree against the oracle's double tree, bit for bit."""
+    from ipc_rank_program import AUTO_SIZES
+    from tccl_amd import ipc
+    world = 8
+    codes, outs = run_ranks(world, tmp_path, "auto", timeout=160)
+    assert codes == [0] * world, "\n".join(outs)
+    picked = dict((tuple(line.split()[1:3]), line.split()[3]) for line in outs[0].splitlines() if line.startswith("PICKED"))
+    assert picked[("small", "auto")] == "one_shot" and picked[("at", "auto")] == "one_shot"
+    assert picked[("above", "auto")] == "two_shot" and picked[("large", "auto")] == "two_shot"
+    for tag, numel in AUTO_SIZES(world, ipc.IpcWorld.ONE_SHOT_MAX_BYTES // 2):
+        bufs = seeded_randn(world, numel)
+        flat = torch_ref.all_reduce(bufs).view(torch.int16)
+        tree = torch_ref.double_tree_all_reduce(bufs)[0].view(torch.int16)
+        for algorithm in ("auto", "one_shot", "two_shot", "double_tree"):
+            want = tree if algorithm == "double_tree" else flat
+            for r in range(world):
+                got = load(tmp_path, f"auto_{tag}.{algorithm}", r, torch.bfloat16).view(torch.int16)
+                assert torch.equal(got, want), f"{tag} {algorithm} rank {r}"
+
+
 @pytest.mark.parametrize("world", [8, 4])
 def test_reference_self_tests_with_a_process_per_rank(world, tmp_path):
     """The `__main__` self-tests of the reference's kernel files (every rank fills its buffer

@@ -608,6 +608,25 @@ def test_tree_reduce_step_large_in_place(_gpu_hygiene, c_oracle):
     assert_bit_equal(d_own, want, "in place, large")
 
 
+@pytest.mark.parametrize("numel", [33_554_432, 33_554_432 + 8 * 1025 + 3], ids=["64MiB", "64MiB-ragged"])
+def test_tree_reduce_step_two_children_in_place_full_tiles(numel, _gpu_hygiene, c_oracle):
+    """64 MiB of output, own + two children, stored over own: the size at which three sources are cut
+    into full 128 KiB tiles and take the kernel whose workgroup pairs share a region in alternate
+    pieces -- each workgroup must have read all its pieces before it writes any.  Also with a ragged
+    end (a partial tile and three elements beyond the last vector).  Children must come out untouched."""
+    torch.manual_seed(7)
+    base = torch.randn(numel, dtype=torch.bfloat16)
+    own, c0, c1 = base, base.roll(9_876_543), base.roll(-3_456_789)
+    want = oracle_sum(c_oracle, [c0, c1, own])
+    d_own, d0, d1 = own.to(DEV), c0.to(DEV), c1.to(DEV)
+    rc = tccl_amd.load_library().tccl_tree_reduce_step(d_own.data_ptr(), d0.data_ptr(), d1.data_ptr(),
+                                                       d_own.data_ptr(), numel, _lib.TCCL_BF16, stream())
+    assert rc == 0
+    assert_bit_equal(d_own, want, "in place, full tiles")
+    assert_bit_equal(d0, c0, "child0 untouched")
+    assert_bit_equal(d1, c1, "child1 untouched")
+
+
 @pytest.mark.parametrize("two", [False, True])
 def test_tree_copy_step(two, _gpu_hygiene):
     src = seeded_int8(1, 16 * 100_003)[0]
