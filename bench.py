@@ -42,6 +42,10 @@ LAT_BYTES_PER_BUF = 1 << 20
 COLD_BYTES = 1 << 30            # a rotation touches at least this much between two uses of a byte (cache: 256 MB)
 MIN_SETS = 4                    # ... over at least this many disjoint buffer sets
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "headline_traffic.json")
+# What a launch of 512 x 256 lanes lasts that loads and stores ONE vector per lane from cold memory (rocprofv3,
+# profiles/probe_kernels_fixed_cost_of_a_short_cold_launch.txt; `bench.py --only floor` measures it again):
+# the part of a short kernel's time that does not depend on its bytes.
+LAUNCH_COST_US = 2.6
 
 ONLY_OPS = ["all_reduce", "all_reduce_rotated", "probe_read", "probe_write", "reduce_scatter_bf16", "reduce_scatter_f32",
             "all_gather_bf16", "all_gather_f32", "all_gather_int8", "tree_reduce_c0", "tree_reduce_c1",
@@ -699,6 +703,8 @@ def other_ops(torch, tccl_amd, lib, plib, noise, device, ceilings=None):
             rd, wr = READS_WRITES[name]
             bound_us = rd / ceilings["read_8_streams_128KiB_tiles_gbs"] / 1e3 + wr / ceilings["write_64MiB_32KiB_tiles_gbs"] / 1e3
             out[name]["of_bound"] = round(bound_us / (ms * 1e3), 3)
+            # the same with the cost of a launch that moves almost nothing taken off the operation's time
+            out[name]["of_bound_beyond_launch_cost"] = round(bound_us / (ms * 1e3 - LAUNCH_COST_US), 3)
         ops.close()
     # whole double-tree all-reduce, W=8 x 256 MiB: level schedule, pipelined single launch (both chunk sizes, both bindings)
     for how, key in (("level", "double_tree_w8_256MiB_level_schedule_ms"),

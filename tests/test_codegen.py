@@ -83,3 +83,22 @@ def test_pipelined_kernel_uses_device_scope_accesses_and_no_cache_flushes(asm):
     assert any(not re.search(r"\bsc1\b", line) for line in loads) and any(re.search(r"\bsc1\b", line) for line in loads)
     assert "buffer_wbl2" not in text and "buffer_inv" not in text
     assert "s_sleep" in text and "global_atomic_add" in text
+    # One launch per rank (the peers are other processes' kernels, which may start and end at any time):
+    # every data load is device-scope, shot 1 of the two-shot kernel included; flags are raised by
+    # device-scope stores and taken by device-scope compare-and-swaps.
+    per_rank = {n: b for n, b in bodies.items() if any(k in n for k in ("sum_rank_kernel", "gather_rank_kernel",
+                                                                        "two_shot_rank_kernel"))}
+    assert len(per_rank) == 16 + 1 + 16
+    for n, body in per_rank.items():
+        loads = re.findall(r"buffer_load_dwordx4[^\n]*", body)
+        stores = re.findall(r"buffer_store_dwordx4[^\n]*", body)
+        assert loads and stores, n
+        assert all(re.search(r"\bsc1\b", line) for line in loads), f"{n}: a data load is not device-scope"
+        assert all(re.search(r"\bsc1\b", line) for line in stores), f"{n}: a data store is not device-scope"
+        if "Li1E" in n and "gather" not in n:
+            continue                          # a world of one has nobody to wait for
+        swaps = re.findall(r"global_atomic_cmpswap[^\n]*", body)
+        raises = re.findall(r"global_store_dword [^\n]*", body)
+        assert swaps, f"{n}: flags are not taken with compare-and-swap"     # (a read-modify-write is carried out beyond the XCD's L2 as it is)
+        assert raises and all(re.search(r"\bsc1\b", line) for line in raises), f"{n}: flags are not raised at device scope"
+        assert body.count("v_readfirstlane_b32") < 64, f"{n}: buffer descriptors are not wave-uniform"
