@@ -71,6 +71,7 @@ def parse_args():
     p.add_argument("--no-other-ops", action="store_true",
                    help="skip reduce-scatter, all-gather, the tree node steps and the signalling kernels")
     p.add_argument("--no-sweep", action="store_true", help="skip the size sweep")
+    p.add_argument("--no-ipc", action="store_true", help="skip the leg with one process per rank")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run 20 plain copies of 256 MiB (tccl_tree_copy_step), so that a rocprofv3 --pmc "
                         "run of this command holds a kernel of known traffic to scale the counters by")
@@ -681,6 +682,75 @@ READS_WRITES = {
 }
 
 
+def cpu_other_ops(torch):
+    """The torch CPU oracle beside two of the other operations, at their benchmark shapes: the all-gather
+    pack (W rows copied into a pre-allocated [W, n]) and the tree node step with two children (fp32
+    accumulate of child0, child1, own, one rounding).  Median of 5 passes after 2 warm-up passes."""
+    from oracle import torch_ref
+    out = {}
+    n = 8_388_608
+    tile = torch.randn(1 << 20, dtype=torch.bfloat16)            # values do not matter to the timing: one MiB-sized tile, repeated
+
+    def noise_of(numel, shift):
+        return tile.roll(shift).repeat(numel // tile.numel())
+
+    # six sets of rows and outputs (1.5 GiB), one per pass: a large host's last-level cache holds one set whole
+    nsets = 6
+    sets = [([noise_of(n, 4099 * r + k) for r in range(WORLD)], torch.zeros((WORLD, n), dtype=torch.bfloat16))
+            for k in range(nsets)]
+    turn = [0]
+
+    def gather():
+        rows, packed = sets[turn[0] % nsets]
+        turn[0] += 1
+        for r in range(WORLD):
+            packed[r].copy_(rows[r])
+
+    def median_s(fn):
+        times = []
+        for i in range(7):
+            t0 = time.perf_counter()
+            fn()
+            if i >= 2:
+                times.append(time.perf_counter() - t0)
+        return statistics.median(times)
+
+    t = median_s(gather)
+    assert torch.equal(sets[0][1].view(torch.int16), torch_ref.all_gather(sets[0][0]).view(torch.int16))
+    out["all_gather_bf16"] = {"cpu_gbs": round(2 * WORLD * n * 2 / t / 1e9, 2), "cpu_ms": round(t * 1e3, 2)}
+    del sets
+    half = 67_108_864
+    own, c0, c1 = (noise_of(half, 7 + 1031 * i) for i in range(3))
+    t = median_s(lambda: torch_ref.tree_reduce_step(own, c0, c1))
+    out["tree_reduce_c2"] = {"cpu_gbs": round(4 * half * 2 / t / 1e9, 2), "cpu_ms": round(t * 1e3, 2)}
+    out["threads"] = torch.get_num_threads()
+    return out
+
+
+def per_process_ranks(seconds=150):
+    """The collectives with every rank a process of its own on this GPU (benchlib/ipc_forms.py, 8 child
+    processes started through python -m tccl_amd.launch): median us per collective of every form at 1,
+    16 and 64 MiB per buffer.  A leg of its own at the very end; whatever goes wrong in it is reported,
+    never raised."""
+    import subprocess
+    cmd = [sys.executable, "-m", "tccl_amd.launch", "--nproc-per-node", "8", "--timeout", str(seconds - 20),
+           os.path.join(ROOT, "benchlib", "ipc_forms.py"), "--json", "--sizes", "1024,16384,65536"]
+    try:
+        done = subprocess.run(cmd, cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=seconds)
+    except subprocess.TimeoutExpired:
+        return {"error": f"no result within {seconds} s"}
+    rows = {}
+    for line in done.stdout.splitlines():
+        if line.startswith('{"ipc_forms"'):
+            rec = json.loads(line)
+            rows[f"{rec['kib_per_buffer'] >> 10}MiB"] = rec["median_us"]
+    if done.returncode != 0 or not rows:
+        return {"error": f"exit code {done.returncode}: {done.stderr.strip()[-300:]}"}
+    rows["note"] = ("8 processes share this GPU, one rank each; median us per collective on rank 0's stream; x3 = barrier launch + "
+                    "kernel + barrier launch, fused = one launch per rank with the barriers inside the kernel")
+    return rows
+
+
 def other_ops(torch, tccl_amd, lib, plib, noise, device, ceilings=None):
     """The other operations of the path at their full benchmark shapes: GB/s on algorithmic bytes
     from HIP events (about 6 ms of launches after a short first pass), every one rotated over enough disjoint buffers
@@ -965,6 +1035,13 @@ def main():
         except RuntimeError as e:        # the headline must still be printed
             result["other_ops"] = {"error": str(e)[:200]}
 
+    if not args.no_cpu_baseline and "error" not in result.get("other_ops", {"error": 1}):
+        # the CPU oracle beside the all-gather pack and the two-children tree step
+        cpu = cpu_other_ops(torch)
+        for name in ("all_gather_bf16", "tree_reduce_c2"):
+            result["other_ops"][name].update(cpu[name])
+        result["other_ops"]["cpu_threads"] = cpu["threads"]
+
     if not args.no_sweep:
         try:
             result["sweep"] = sweep(torch, tccl_amd, lib, noise, device)
@@ -973,6 +1050,11 @@ def main():
 
     if args.calibrate_copy:
         calibrate_copy(torch, lib, device)
+
+    if not args.no_ipc and not args.no_other_ops:
+        free(torch)
+        torch.cuda.synchronize()
+        result["per_process_ranks"] = per_process_ranks()
 
     print(json.dumps(result), flush=True)
 

@@ -1,6 +1,6 @@
 """What the collectives cost when every rank is a process of its own on the one GPU, form by form:
 
-    python -m tccl_amd.launch --nproc-per-node 8 benchlib/ipc_forms.py
+    python -m tccl_amd.launch --nproc-per-node 8 benchlib/ipc_forms.py [--json] [--sizes KiB,KiB,...]
 
 Per buffer size rank 0 prints the time per collective (HIP events on its own stream, all ranks in
 step: the median and, in brackets, the fastest of 5 blocks of 16 calls after 8 warm-up calls) of
@@ -16,8 +16,11 @@ step: the median and, in brackets, the fastest of 5 blocks of 16 calls after 8 w
 
 The in-place forms rescale the buffer before every call so that values stay finite; that small
 kernel is part of their time.  On one GPU the W processes' queues take turns, so these times say how
-the forms compare with each other here, not what they would cost with a GPU per rank."""
+the forms compare with each other here, not what they would cost with a GPU per rank.
+``--json``: one JSON line per size instead of the table (bench.py reads those); ``--sizes``: buffer sizes
+in KiB instead of 64 KiB ... 256 MiB."""
 import ctypes
+import json
 import os
 import sys
 
@@ -28,7 +31,15 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 from tccl_amd import _lib, ipc        # noqa: E402
 
 
+COLUMNS = ("barrier", "one_shot_x3", "one_shot_fused", "reduce_scatter_x3", "reduce_scatter_fused", "all_gather_x3",
+           "all_gather_fused", "two_shot_x3", "two_shot_fused", "double_tree_x3")
+
+
 def main() -> int:
+    as_json = "--json" in sys.argv
+    sizes = (64, 1024, 4096, 16384, 65536, 262144)
+    if "--sizes" in sys.argv:
+        sizes = tuple(int(v) for v in sys.argv[sys.argv.index("--sizes") + 1].split(","))
     world = ipc.IpcWorld.from_env()
     rank, size = world.rank, world.world_size
     lib = world.lib
@@ -47,13 +58,16 @@ def main() -> int:
         torch.cuda.synchronize()
         world.check()
         us = sorted(ev[b].elapsed_time(ev[b + 1]) * 1000 / reps for b in range(blocks))
-        return f"{us[blocks // 2]:.0f} ({us[0]:.0f})"
+        return us[blocks // 2], us[0]
 
-    if rank == 0:
+    def show(pair):
+        return "-" if pair is None else f"{pair[0]:.0f} ({pair[1]:.0f})"
+
+    if rank == 0 and not as_json:
         print(f"{size} processes on one GPU; us per collective on rank 0's stream", flush=True)
         print(f"{'per buffer':>10s} {'barrier':>10s} | {'one-shot x3':>11s} {'fused':>11s} | {'rs x3':>10s} {'fused':>10s} | "
               f"{'ag x3':>10s} {'fused':>10s} | {'two-shot x3':>11s} {'fused':>11s} | {'tree':>11s}", flush=True)
-    for kib in (64, 1024, 4096, 16384, 65536, 262144):
+    for kib in sizes:
         numel = kib << 9
         t = world.empty(numel, torch.bfloat16)
         t.copy_(torch.randn(numel, dtype=torch.bfloat16) * 0.01)
@@ -75,16 +89,20 @@ def main() -> int:
 
         us = [timed(world.barrier)]
         us.append(timed(between_barriers(lambda: lib.tccl_all_reduce_sum(ptrs, size, out.data_ptr(), numel, 0, stream()))))
-        us.append(timed(lambda: world.one_shot_all_reduce(t, out=out)))
+        us.append(timed(lambda: world.one_shot_all_reduce(t, out=out, fused=True)))
         us.append(timed(between_barriers(lambda: lib.tccl_reduce_scatter_sum(ptrs, size, rank, share.data_ptr(), numel, 0, stream()))))
-        us.append(timed(lambda: world.reduce_scatter(t, out=share)))
+        us.append(timed(lambda: world.reduce_scatter(t, out=share, fused=True)))
         us.append(timed(between_barriers(lambda: lib.tccl_all_gather(ptrs, size, gathered.data_ptr(), part.numel() * 2, stream()))))
-        us.append(timed(lambda: world.all_gather(part, out=gathered)))
+        us.append(timed(lambda: world.all_gather(part, out=gathered, fused=True)))
         us.append(timed(lambda: (t.mul_(1.0 / size), world.two_shot_all_reduce(t, own_barriers=False))))
         us.append(timed(lambda: (t.mul_(1.0 / size), world.two_shot_all_reduce(t))))
-        us.append(timed(lambda: (t.mul_(1.0 / size), world.double_tree_all_reduce(t))) if size in (2, 4, 8) else "-")
-        if rank == 0:
+        us.append(timed(lambda: (t.mul_(1.0 / size), world.double_tree_all_reduce(t))) if size in (2, 4, 8) else None)
+        if rank == 0 and as_json:
+            print(json.dumps({"ipc_forms": True, "processes": size, "kib_per_buffer": kib,
+                              "median_us": {c: None if p is None else round(p[0], 1) for c, p in zip(COLUMNS, us)}}), flush=True)
+        elif rank == 0:
             label = f"{kib} KiB" if kib < 1024 else f"{kib >> 10} MiB"
+            us = [show(p) for p in us]
             print(f"{label:>10s} {us[0]:>10s} | {us[1]:>11s} {us[2]:>11s} | {us[3]:>10s} {us[4]:>10s} | "
                   f"{us[5]:>10s} {us[6]:>10s} | {us[7]:>11s} {us[8]:>11s} | {us[9]:>11s}", flush=True)
     world.close()
