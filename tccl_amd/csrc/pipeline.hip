@@ -510,32 +510,28 @@ static size_t workgroups_per_rank(size_t units, size_t most, int world, bool tie
 // a signalling grid of 8 per unit once timed out for a reason that was never established, so
 // that shape stays unreachable whatever a kernel's register use becomes.
 //
-// waits_at_entry: the kernel's workgroups wait for their peers before they do anything (a
-// leading barrier), and the peers' launches may arrive much later, behind other kernels.  Then
-// the occupancy the runtime reports cannot be relied on: a wave's registers are one contiguous
-// block of its SIMD's 512, short-lived waves of other kernels that come and go between the
-// arrivals leave the waiting waves scattered over the file, and the holes between them may each
-// be too small for the late launch's waves although their sum is not.  (Measured with 8
-// processes at the reported 4 per unit: the last rank's launch got 2 of its 128 workgroups
-// placed and the other 896 waited for it until their waits expired.)  With n waves of v
+// separate_launches: the workgroups that wait for each other belong to different launches (one
+// per rank, from different processes), which arrive at different times behind other kernels.  Then
+// the occupancy the runtime reports cannot be relied on.  Measured with 8 processes at the
+// reported 4 per unit, each rank's collective behind an elementwise kernel of its own: the last
+// rank's launch got 2 of its 128 workgroups placed, and the other 896, which left room for 126
+// more by the runtime's count, waited for the rest until their waits expired.  The explanation
+// that fits: a wave's registers are one contiguous block of its SIMD's 512, the short-lived waves
+// of the other kernels that come and go between the arrivals leave the waiting waves scattered
+// over the file, and the holes between them may each be too small for the late launch's waves
+// although their sum is not.  With n waves of v
 // registers per SIMD wanted, n - 1 badly placed ones leave a hole of at least
 // (512 - (n - 1) v) / n, which holds the n-th for n <= (512 + v) / (2 v): half the reported
 // figure, rounded up.  Only as many workgroups as that are launched, so the last arrival
 // always finds room.
 template <class K>
-static int resident_for(K kernel, bool waits_at_entry = false)
+static int resident_for(K kernel, bool separate_launches = false)
 {
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kPhasedBlock, 0) != hipSuccess || per_cu < 1) return 0;
     if (per_cu > kMaxSignallingPerUnit) per_cu = kMaxSignallingPerUnit;
-    if (waits_at_entry) per_cu = (per_cu + 1) / 2;
+    if (separate_launches) per_cu = (per_cu + 1) / 2;
     return per_cu * compute_units();
-}
-
-template <class Sum, int VECS>
-static int resident_workgroups()
-{
-    return resident_for(tree_pipelined_kernel<Sum, VECS>);
 }
 
 template <class Sum, int VECS>
@@ -543,9 +539,14 @@ static int launch_pipelined(const PipeArgs &a, int wgs_wanted, int world, size_t
 {
     // asked once per kernel: the answer depends on the kernel's register use only
     static std::once_flag once;
-    static int resident = 0;
-    std::call_once(once, [] { resident = resident_workgroups<Sum, VECS>(); });
-    // Every workgroup must be resident: the grid never exceeds what the runtime says fits.
+    static int resident_one = 0, resident_per_rank = 0;
+    std::call_once(once, [] {
+        resident_one = resident_for(tree_pipelined_kernel<Sum, VECS>);
+        resident_per_rank = resident_for(tree_pipelined_kernel<Sum, VECS>, true);
+    });
+    // Every workgroup must be resident: the grid never exceeds what the runtime says fits -- or, where
+    // the ranks' launches come from different processes at different times, what always finds room.
+    const int resident = a.only_rank >= 0 ? resident_per_rank : resident_one;
     if (resident < world) return hip_code(hipErrorLaunchOutOfResources);
     int per_rank;
     if (wgs_wanted > 0) {
@@ -894,13 +895,12 @@ template <class Sum, int W>
 static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, const ClearRequest *clear, hipStream_t s)
 {
     static std::once_flag once;
-    static int resident_one = 0, resident_rank = 0, resident_rank_entry = 0;
+    static int resident_one = 0, resident_rank = 0;
     std::call_once(once, [] {
         resident_one = resident_for(two_shot_kernel<Sum, W>);
-        resident_rank = resident_for(two_shot_rank_kernel<Sum, W>);
-        resident_rank_entry = resident_for(two_shot_rank_kernel<Sum, W>, true);
+        resident_rank = resident_for(two_shot_rank_kernel<Sum, W>, true);
     });
-    const int resident = a.only_rank < 0 ? resident_one : (a.own_barriers ? resident_rank_entry : resident_rank);
+    const int resident = a.only_rank < 0 ? resident_one : resident_rank;
     if (resident < W) return hip_code(hipErrorLaunchOutOfResources);
     constexpr size_t tile_bytes = static_cast<size_t>(kPhasedBlock) * kTwoShotVecs * kVecBytes;
     const size_t tiles = (a.share_bytes + tile_bytes - 1) / tile_bytes;
