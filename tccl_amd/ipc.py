@@ -263,9 +263,9 @@ class IpcWorld:
     # bytes, and barrier launch + the library's full-size kernel + barrier launch above: a rank's own launch
     # holds only 1/W of the workgroups that are certain to find room beside the peers' launches and works in
     # 16 KiB tiles, which costs more than two extra launches once the data is large (8 processes on one
-    # MI355X, all-reduce of 8 x 16 MiB = 144 MiB moved: 298-313 us fused against 287-328 us; 8 x 64 MiB:
-    # 1,110 against 880-900 us; reduce-scatter of 8 x 256 MiB = 288 MiB moved: 560 against 460-500 us, of
-    # 8 x 64 MiB = 72 MiB: 172-183 against 199-233 us; profiles/ipc_forms_one_gpu_8_4_2_processes.txt).
+    # MI355X, all-reduce of 8 x 16 MiB = 144 MiB moved: 289-306 us fused against 302-326 us; 8 x 64 MiB:
+    # 1,097-1,119 against 881-891 us; reduce-scatter of 8 x 256 MiB = 288 MiB moved: 556-571 against 474-502 us, of
+    # 8 x 64 MiB = 72 MiB: 167-183 against 201-237 us; profiles/ipc_forms_one_gpu_8_4_2_processes.txt).
     FUSED_MAX_MOVED_BYTES = 128 << 20
 
     def _one_shot(self, name: str, tensor: torch.Tensor, out: torch.Tensor, size_arg: int, with_dtype: bool,
@@ -348,10 +348,10 @@ class IpcWorld:
     # all_reduce(algorithm="auto"): one-shot up to this many bytes per buffer, two-shot above it in worlds of more
     # than 4.  Measured with 8 processes on one MI355X (python -m tccl_amd.launch --nproc-per-node 8
     # benchlib/ipc_forms.py, us per collective, one-shot / two-shot / double tree; profiles/
-    # ipc_forms_one_gpu_8_4_2_processes.txt): 1 MiB 58-72 / 139-184 / 236-310; 4 MiB 105-118 / 162-203 / 267-341;
-    # 16 MiB 287-313 / 244-287 / 339-413; 64 MiB 880-900 / 700-730 / 850-925; 256 MiB 3,300 / 2,600-2,790 /
-    # 2,880-2,990.  With 4 processes (and with 2) the one-shot form is the fastest at every size: 64 MiB
-    # 264-269 / 311 / 386, 256 MiB 923 / 1,250 / 1,245; worlds of 5 to 7 were not measured and take the rule
+    # ipc_forms_one_gpu_8_4_2_processes.txt): 1 MiB 55-69 / 140-178 / 252-319; 4 MiB 98-113 / 162-197 / 281-347;
+    # 16 MiB 289-326 / 244-275 / 363-430; 64 MiB 881-891 / 729-745 / 932-974; 256 MiB 3,300 / 2,762-2,931 /
+    # 3,218-3,241.  With 4 processes (and with 2) the one-shot form is the fastest at every size: 64 MiB
+    # 263-270 / 309 / 408, 256 MiB 922 / 1,261 / 1,324; worlds of 5 to 7 were not measured and take the rule
     # of 8.  The double tree is never the fastest on one GPU and is run by name only.  Across GPUs the
     # one-shot form moves W - 1 whole buffers per rank over the links and the thresholds would sit far lower.
     ONE_SHOT_MAX_BYTES = 8 << 20
