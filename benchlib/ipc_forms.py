@@ -12,7 +12,7 @@ step: the median and, in brackets, the fastest of 5 blocks of 16 calls after 8 w
   ag x3 / ag fused    ... and of the all-gather (every rank contributes 1/W of the buffer size)
   two-shot x3 / fused barrier + tccl_two_shot_all_reduce_rank + barrier, and the same kernel with
                       TCCL_PIPE_OWN_BARRIERS: one launch per rank (both in place)
-  tree                barrier + tccl_double_tree_all_reduce_pipelined_rank + barrier (in place)
+  tree x3 / fused     the same two forms of tccl_double_tree_all_reduce_pipelined_rank (in place)
 
 The in-place forms rescale the buffer before every call so that values stay finite; that small
 kernel is part of their time.  On one GPU the W processes' queues take turns, so these times say how
@@ -32,7 +32,7 @@ from tccl_amd import _lib, ipc        # noqa: E402
 
 
 COLUMNS = ("barrier", "one_shot_x3", "one_shot_fused", "reduce_scatter_x3", "reduce_scatter_fused", "all_gather_x3",
-           "all_gather_fused", "two_shot_x3", "two_shot_fused", "double_tree_x3")
+           "all_gather_fused", "two_shot_x3", "two_shot_fused", "double_tree_x3", "double_tree_fused")
 
 
 def main() -> int:
@@ -66,7 +66,7 @@ def main() -> int:
     if rank == 0 and not as_json:
         print(f"{size} processes on one GPU; us per collective on rank 0's stream", flush=True)
         print(f"{'per buffer':>10s} {'barrier':>10s} | {'one-shot x3':>11s} {'fused':>11s} | {'rs x3':>10s} {'fused':>10s} | "
-              f"{'ag x3':>10s} {'fused':>10s} | {'two-shot x3':>11s} {'fused':>11s} | {'tree':>11s}", flush=True)
+              f"{'ag x3':>10s} {'fused':>10s} | {'two-shot x3':>11s} {'fused':>11s} | {'tree x3':>11s} {'fused':>11s}", flush=True)
     for kib in sizes:
         numel = kib << 9
         t = world.empty(numel, torch.bfloat16)
@@ -96,7 +96,9 @@ def main() -> int:
         us.append(timed(lambda: world.all_gather(part, out=gathered, fused=True)))
         us.append(timed(lambda: (t.mul_(1.0 / size), world.two_shot_all_reduce(t, own_barriers=False))))
         us.append(timed(lambda: (t.mul_(1.0 / size), world.two_shot_all_reduce(t))))
-        us.append(timed(lambda: (t.mul_(1.0 / size), world.double_tree_all_reduce(t))) if size in (2, 4, 8) else None)
+        trees = size in (2, 4, 8)
+        us.append(timed(lambda: (t.mul_(1.0 / size), world.double_tree_all_reduce(t, own_barriers=False))) if trees else None)
+        us.append(timed(lambda: (t.mul_(1.0 / size), world.double_tree_all_reduce(t))) if trees else None)
         if rank == 0 and as_json:
             print(json.dumps({"ipc_forms": True, "processes": size, "kib_per_buffer": kib,
                               "median_us": {c: None if p is None else round(p[0], 1) for c, p in zip(COLUMNS, us)}}), flush=True)
@@ -104,7 +106,7 @@ def main() -> int:
             label = f"{kib} KiB" if kib < 1024 else f"{kib >> 10} MiB"
             us = [show(p) for p in us]
             print(f"{label:>10s} {us[0]:>10s} | {us[1]:>11s} {us[2]:>11s} | {us[3]:>10s} {us[4]:>10s} | "
-                  f"{us[5]:>10s} {us[6]:>10s} | {us[7]:>11s} {us[8]:>11s} | {us[9]:>11s}", flush=True)
+                  f"{us[5]:>10s} {us[6]:>10s} | {us[7]:>11s} {us[8]:>11s} | {us[9]:>11s} {us[10]:>11s}", flush=True)
     world.close()
     return 0
 

@@ -257,8 +257,8 @@ typedef struct {
 } tccl_pipeline_cfg;
 
 #define TCCL_PIPE_DRAW_PLACES 1 /* workgroups draw their places when they start (see above) */
-#define TCCL_PIPE_OWN_BARRIERS 2 /* tccl_two_shot_all_reduce_rank only: the kernel begins and ends with the
-                                    blockwise barrier itself (see there) */
+#define TCCL_PIPE_OWN_BARRIERS 2 /* tccl_two_shot_all_reduce_rank and tccl_double_tree_all_reduce_pipelined_rank:
+                                    the kernel begins and ends with the blockwise barrier itself (see there) */
 
 size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int dtype, size_t chunk_elems);
 int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs,
@@ -275,9 +275,12 @@ int tccl_double_tree_all_reduce_pipelined(void *const *bufs, void *const *outs,
  * at the same time (each holds 1/world of the workgroups that fit the GPU) and must all be given
  * the same numel, dtype, chunk_elems and cfg.  Between two collectives on the same buffers and
  * pads every rank must have finished the first before any rank starts the second (and the inputs
- * must be in place before any rank starts): tccl_blockwise_barrier() before and after, as the
- * reference begins its kernels with blockwise_barrier.  TCCL_PIPE_DRAW_PLACES does not apply
- * (TCCL_EINVAL).  Time-outs, pads, chunking, arithmetic: as above. */
+ * must be in place before any rank starts): either TCCL_PIPE_OWN_BARRIERS in cfg->flags -- the
+ * kernel then begins with the blockwise barrier, as the reference's does
+ * (triton_double_tree_allreduce.py:239), and ends with one, on slots of their own behind the
+ * chunks' (the size tccl_double_tree_signal_pad_bytes() returns has room for them; at most 512
+ * workgroups per rank) -- or tccl_blockwise_barrier() before and after.  TCCL_PIPE_DRAW_PLACES does
+ * not apply (TCCL_EINVAL).  Time-outs, pads, chunking, arithmetic: as above. */
 int tccl_double_tree_all_reduce_pipelined_rank(void *const *bufs, void *out, void *const *signal_pads,
                                                size_t pad_bytes, int world, int rank, size_t numel,
                                                int dtype, size_t chunk_elems,

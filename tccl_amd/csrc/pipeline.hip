@@ -48,6 +48,9 @@ constexpr uint32_t kPipeDefaultSpins = 1u << 21;
 // Most workgroups per compute unit a grid whose workgroups wait for each other may have (see
 // resident_for).
 constexpr int kMaxSignallingPerUnit = 6;
+// Most workgroups per rank of a per-rank launch of the double tree that carries its own barriers
+// (its pads have two rows of barrier slots for that many).
+constexpr size_t kTreeBarrierWorkgroups = 512;
 
 // Two signalling kernels that overlap on one GPU could each hold part of the workgroup slots
 // and (with places bound by hardware index) starve each other until their waits expire; with
@@ -116,6 +119,8 @@ struct PipeArgs {
     int world, wgs_per_rank, lag, tree_height;
     int draw;         // 1 = workgroups draw their places when they start, 0 = places follow the hardware index
     int only_rank;    // >= 0: the launch holds this rank's workgroups only (one launch per rank); -1: all ranks'
+    int own_barriers; // one launch per rank: the kernel also begins and ends with the blockwise barrier
+    uint32_t barrier_base; // first word of the barriers' slots in a pad (behind the chunk slots)
     uint32_t *ctl;    // the control words at the end of pad 0 (place counters ... time-outs)
     uint32_t *report; // optional word in host memory that is set to 1 when a wait expires
 };
@@ -284,6 +289,32 @@ __device__ __forceinline__ bool wait_signals(uint32_t *slot0, uint32_t *slot1, u
     return ok != 0;
 }
 
+// The reference's blockwise barrier (triton_barrier.py:39-142) between the workgroups with the
+// same index of all W ranks, on the W slots that start at word `base` of every pad: lane i < W of
+// the first wave raises slot `base + rank` in rank i's pad and takes slot `base + i` of the own
+// pad (each slot has one writer and one reader, so the sender's compare-and-swap 0 -> 1 of the
+// reference becomes a plain store; the wait is its compare-and-swap 1 -> 0, take_flag).
+// Everything the workgroup stored before the barrier is visible to its peers' device-scope loads
+// after it.  *lds_ok must be 1 on entry; returns false when a wait expired (counted in the
+// control words).
+__device__ __forceinline__ bool barrier_on_slots(uint32_t *const *pad, int world, int rank, uint32_t base,
+                                                 uint32_t spin_limit, uint32_t *ctl, uint32_t *report, int *lds_ok)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const int lane = threadIdx.x;
+    if (lane < world && lane != rank) {
+        __hip_atomic_store(pad[lane] + base + rank, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t spent = 0;
+        if (!take_flag(pad[rank] + base + lane, spin_limit, &spent)) {
+            report_timeout(ctl, report);
+            *lds_ok = 0; // any lane that failed clears the flag
+        }
+    }
+    __syncthreads();
+    return *lds_ok != 0;
+}
+
 // One chunk of a reduce step: sources -> destinations, in tiles of VECS vectors per lane
 // (256 lanes: 32 KiB for VECS = 8, 128 KiB for VECS = 32), each read and reduced into
 // registers and then written.
@@ -402,7 +433,20 @@ __device__ __forceinline__ void tree_pipelined_walk(const PipeArgs &a, int rank,
 {
     const uint32_t G = a.wgs_per_rank;
     const uint32_t most = a.nchunks[0] > a.nchunks[1] ? a.nchunks[0] : a.nchunks[1];
-    if (g >= most) return;
+    if (g >= most) return; // (the same workgroups in every rank's launch)
+    // One launch per rank with the reference's leading barrier inside (the double tree's kernel
+    // begins with blockwise_barrier, triton_double_tree_allreduce.py:239): every rank's input is
+    // in place before anybody reads a leaf's buffer.  The trailing barrier (row G + g) tells the
+    // peers that this workgroup has taken every flag and read every chunk it ever will, so buffers
+    // and pads are free for the next collective when the kernel has ended.  Two rows in turn, as
+    // in the one-shot kernels.
+    const bool own_barriers = a.only_rank >= 0 && a.own_barriers != 0;
+    if (own_barriers) {
+        if (threadIdx.x == 0) *lds_ok = 1;
+        if (!barrier_on_slots(a.pad, a.world, rank, a.barrier_base + g * a.world, a.spin_limit, a.ctl, a.report, lds_ok))
+            return;
+        __syncthreads(); // wait_signals rewrites lds_ok
+    }
     const uint32_t rounds = (most - g + G - 1) / G;
     const uint32_t lag = a.lag;
     for (uint32_t i = 0; i < rounds + lag; ++i) {
@@ -416,6 +460,11 @@ __device__ __forceinline__ void tree_pipelined_walk(const PipeArgs &a, int rank,
             for (int t = 0; t < 2; ++t)
                 if (c < a.nchunks[t] && !down_step<VECS>(a, rank, t, c, lds_ok)) return;
         }
+    }
+    if (own_barriers) {
+        __syncthreads();
+        if (threadIdx.x == 0) *lds_ok = 1;
+        (void)barrier_on_slots(a.pad, a.world, rank, a.barrier_base + (G + g) * a.world, a.spin_limit, a.ctl, a.report, lds_ok);
     }
 }
 
@@ -556,6 +605,7 @@ static int launch_pipelined(const PipeArgs &a, int wgs_wanted, int world, size_t
     } else {
         per_rank = static_cast<int>(workgroups_per_rank(slots, static_cast<size_t>(resident / world), world, true));
     }
+    if (a.own_barriers && static_cast<size_t>(per_rank) > kTreeBarrierWorkgroups) per_rank = static_cast<int>(kTreeBarrierWorkgroups);
     PipeArgs args = a;
     args.wgs_per_rank = per_rank;
     SignallingLaunch guard(s);
@@ -622,8 +672,10 @@ extern "C" size_t tccl_double_tree_signal_pad_bytes(int world, size_t numel, int
 {
     PipeGeometry g;
     if (pipe_geometry(world, numel, dtype, chunk_elems, &g) != TCCL_OK) return 0;
-    // two trees x slots x world flags, then the control words; rounded up to 16 bytes
-    const size_t words = 2 * g.slots * static_cast<size_t>(world) + kCtlWords;
+    // two trees x slots x world flags, two rows of barrier slots for up to kTreeBarrierWorkgroups
+    // workgroups per rank (used by the per-rank launch with TCCL_PIPE_OWN_BARRIERS), then the control
+    // words; rounded up to 16 bytes
+    const size_t words = (2 * g.slots + 2 * kTreeBarrierWorkgroups) * static_cast<size_t>(world) + kCtlWords;
     return (words * sizeof(uint32_t) + 15) / 16 * 16;
 }
 
@@ -674,6 +726,8 @@ static int pipelined_double_tree(void *const *bufs, void *const *outs, void *con
     a.slots = static_cast<uint32_t>(g.slots);
     a.world = world;
     a.only_rank = only_rank;
+    a.own_barriers = (only_rank >= 0 && cfg && (cfg->flags & TCCL_PIPE_OWN_BARRIERS)) ? 1 : 0;
+    a.barrier_base = static_cast<uint32_t>(2 * g.slots * static_cast<size_t>(world));
     a.draw = (only_rank < 0 && cfg && (cfg->flags & TCCL_PIPE_DRAW_PLACES)) ? 1 : 0;
     a.ctl = a.pad[0] + pad_bytes / sizeof(uint32_t) - kCtlWords; // the last words of pad 0
     a.report = cfg ? cfg->timeout_flag : nullptr;
@@ -738,32 +792,10 @@ struct TwoShotArgs {
     uint32_t *report; // optional host word set to 1 when a wait expires
 };
 
-// The reference's blockwise barrier (triton_barrier.py:39-142) between the workgroups with
-// the same index g of all W virtual ranks: lane i < W of the first wave raises slot
-// `g * W + rank` in rank i's pad and waits for slot `g * W + i` in the own pad, which it
-// lowers again (each slot has one writer and one reader, so the sender's compare-and-swap 0 -> 1
-// of the reference becomes a plain store; the wait is the reference's compare-and-swap 1 -> 0,
-// take_flag).  Everything the workgroup stored before the
-// barrier is visible to its peers' device-scope loads after it.  Returns false when a wait
-// expired (counted in the control words).
+// The blockwise barrier of workgroup g on row `row` of the pads (barrier_on_slots).
 __device__ __forceinline__ bool blockwise_barrier(const TwoShotArgs &a, int rank, uint32_t row, int *lds_ok)
 {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    const int lane = threadIdx.x;
-    if (lane < a.world && lane != rank) {
-        const uint32_t base = row * static_cast<uint32_t>(a.world);
-        __hip_atomic_store(a.pad[lane] + base + rank, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t *mine = a.pad[rank] + base + lane;
-        uint32_t polls = 0;
-        const bool ok = take_flag(mine, a.spin_limit, &polls);
-        if (!ok) {
-            report_timeout(a.ctl, a.report);
-            *lds_ok = 0; // any lane that failed clears the flag
-        }
-    }
-    __syncthreads();
-    return *lds_ok != 0;
+    return barrier_on_slots(a.pad, a.world, rank, row * static_cast<uint32_t>(a.world), a.spin_limit, a.ctl, a.report, lds_ok);
 }
 
 // Rank r's workgroup g of G:
@@ -1074,21 +1106,7 @@ struct RankArgs {
 // rank's launch, on row `row` of the pads.
 __device__ __forceinline__ bool rank_barrier(const RankArgs &a, uint32_t row, int *lds_ok)
 {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    const int lane = threadIdx.x;
-    if (lane < a.world && lane != a.rank) {
-        const uint32_t base = row * static_cast<uint32_t>(a.world);
-        __hip_atomic_store(a.pad[lane] + base + a.rank, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t *mine = a.pad[a.rank] + base + lane;
-        uint32_t polls = 0;
-        const bool ok = take_flag(mine, a.spin_limit, &polls);
-        if (!ok)
-            report_timeout(a.ctl, a.report);
-        if (!ok) *lds_ok = 0;
-    }
-    __syncthreads();
-    return *lds_ok != 0;
+    return barrier_on_slots(a.pad, a.world, a.rank, row * static_cast<uint32_t>(a.world), a.spin_limit, a.ctl, a.report, lds_ok);
 }
 
 // 16 KiB tiles, as in the two-shot kernel: a rank has 1/W of the GPU's workgroup slots, and

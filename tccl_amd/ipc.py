@@ -230,18 +230,21 @@ class IpcWorld:
         return out
 
     def double_tree_all_reduce(self, tensor: torch.Tensor, chunk_elems: int = 0,
-                               cfg: Optional[_lib.PipelineCfg] = None) -> torch.Tensor:
+                               cfg: Optional[_lib.PipelineCfg] = None, own_barriers: bool = True) -> torch.Tensor:
         """The reference's double-tree all-reduce as it runs it (triton_double_tree_allreduce.py:338-370):
         this rank's own launch of the pipelined kernel, meeting the other ranks' launches through
-        wait/send on signal pads in each other's memory, between a leading and a trailing barrier.
-        Collective; the symmetric buffers are overwritten (every rank's ends up holding the sum,
-        which is also returned).  Worlds of 2, 4 and 8."""
+        wait/send on signal pads in each other's memory; the kernel begins with the blockwise barrier
+        as the reference's does (:239) and ends with one (``own_barriers=False``: a barrier launch
+        before and after instead).  Collective; the symmetric buffers are overwritten (every rank's
+        ends up holding the sum, which is also returned).  Worlds of 2, 4 and 8."""
         _, _, dtype = self._tables[self._base(tensor)]
         code = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype]
         need = self.lib.tccl_double_tree_signal_pad_bytes(self.world_size, tensor.numel(), code, chunk_elems)
         if need == 0:
             raise ValueError("the pipelined double tree takes worlds of 2, 4 or 8 and whole 16-byte vectors")
-        return self._own_launch("tccl_double_tree_all_reduce_pipelined_rank", tensor, need, (chunk_elems,), cfg)
+        if tensor.numel() == 0:
+            return torch.empty_like(tensor)
+        return self._own_launch("tccl_double_tree_all_reduce_pipelined_rank", tensor, need, (chunk_elems,), cfg, own_barriers)
 
     def two_shot_all_reduce(self, tensor: torch.Tensor, cfg: Optional[_lib.PipelineCfg] = None,
                             own_barriers: bool = True) -> torch.Tensor:
@@ -263,9 +266,9 @@ class IpcWorld:
     # bytes, and barrier launch + the library's full-size kernel + barrier launch above: a rank's own launch
     # holds only 1/W of the workgroups that are certain to find room beside the peers' launches and works in
     # 16 KiB tiles, which costs more than two extra launches once the data is large (8 processes on one
-    # MI355X, all-reduce of 8 x 16 MiB = 144 MiB moved: 289-306 us fused against 302-326 us; 8 x 64 MiB:
-    # 1,097-1,119 against 881-891 us; reduce-scatter of 8 x 256 MiB = 288 MiB moved: 556-571 against 474-502 us, of
-    # 8 x 64 MiB = 72 MiB: 167-183 against 201-237 us; profiles/ipc_forms_one_gpu_8_4_2_processes.txt).
+    # MI355X, all-reduce of 8 x 16 MiB = 144 MiB moved: 292-298 us fused against 290-345 us; 8 x 64 MiB:
+    # 1,024-1,114 against 871-915 us; reduce-scatter of 8 x 256 MiB = 288 MiB moved: 526-559 against 463-521 us, of
+    # 8 x 64 MiB = 72 MiB: 172-175 against 200-250 us; profiles/ipc_forms_one_gpu_8_4_2_processes.txt).
     FUSED_MAX_MOVED_BYTES = 128 << 20
 
     def _one_shot(self, name: str, tensor: torch.Tensor, out: torch.Tensor, size_arg: int, with_dtype: bool,
@@ -348,10 +351,10 @@ class IpcWorld:
     # all_reduce(algorithm="auto"): one-shot up to this many bytes per buffer, two-shot above it in worlds of more
     # than 4.  Measured with 8 processes on one MI355X (python -m tccl_amd.launch --nproc-per-node 8
     # benchlib/ipc_forms.py, us per collective, one-shot / two-shot / double tree; profiles/
-    # ipc_forms_one_gpu_8_4_2_processes.txt): 1 MiB 55-69 / 140-178 / 252-319; 4 MiB 98-113 / 162-197 / 281-347;
-    # 16 MiB 289-326 / 244-275 / 363-430; 64 MiB 881-891 / 729-745 / 932-974; 256 MiB 3,300 / 2,762-2,931 /
-    # 3,218-3,241.  With 4 processes (and with 2) the one-shot form is the fastest at every size: 64 MiB
-    # 263-270 / 309 / 408, 256 MiB 922 / 1,261 / 1,324; worlds of 5 to 7 were not measured and take the rule
+    # ipc_forms_one_gpu_8_4_2_processes.txt): 1 MiB 59-73 / 141-186 / 167-213; 4 MiB 104-122 / 162-226 / 196-242;
+    # 16 MiB 290-345 / 247-310 / 282-327; 64 MiB 871-915 / 705-765 / 834-880; 256 MiB 3,300 / 2,759-2,826 /
+    # 3,140-3,211.  With 4 processes (and with 2) the one-shot form is the fastest at every size: 64 MiB
+    # 206-245 / 272 / 317, 256 MiB 863 / 1,232 / 1,227; worlds of 5 to 7 were not measured and take the rule
     # of 8.  The double tree is never the fastest on one GPU and is run by name only.  Across GPUs the
     # one-shot form moves W - 1 whole buffers per rank over the links and the thresholds would sit far lower.
     ONE_SHOT_MAX_BYTES = 8 << 20

@@ -302,7 +302,8 @@ def main():
                     t.copy_(torch.randn(numel, dtype=dtype))
                 else:
                     t.copy_(torch.rand(numel, dtype=dtype) * 2 - 1)
-                out = world.double_tree_all_reduce(t)
+                # round 0: one launch per rank, the kernel's own barriers; round 1: a barrier launch either side
+                out = world.double_tree_all_reduce(t, own_barriers=(round_ == 0))
                 world.check()
                 save(directory, f"double_tree_{tag}.{round_}.out", rank, out)
                 save(directory, f"double_tree_{tag}.{round_}.buf", rank, t)
