@@ -112,7 +112,7 @@ def test_two_shot_one_launch_per_rank(world, tmp_path):
                     assert torch.equal(got, want), f"{tag} round {round_} rank {r} {what}"
 
 
-@pytest.mark.parametrize("world", [4, 8])
+@pytest.mark.parametrize("world", [3, 4, 8])
 def test_one_shot_kernels_with_their_barriers_inside(world, tmp_path):
     """The reference's form for process-owned ranks (triton_one_shot_all_reduce_no_128.py:46,
     triton_all_gather.py:43): every rank's all-reduce, reduce-scatter and all-gather is ONE launch that
