@@ -302,7 +302,7 @@ def main():
                     t.copy_(torch.randn(numel, dtype=dtype))
                 else:
                     t.copy_(torch.rand(numel, dtype=dtype) * 2 - 1)
-                # round 0: one launch per rank, the kernel's own barriers; round 1: a barrier launch either side
+                # first pass: one launch per rank, the kernel's own barriers; second pass: a barrier launch either side
                 out = world.double_tree_all_reduce(t, own_barriers=(round_ == 0))
                 world.check()
                 save(directory, f"double_tree_{tag}.{round_}.out", rank, out)
@@ -324,7 +324,7 @@ def main():
                     t.copy_(torch.randn(numel, dtype=dtype))
                 else:
                     t.copy_(torch.rand(numel, dtype=dtype) * 2 - 1)
-                # round 0: one launch per rank, the kernel's own barriers; round 1: a barrier launch either side
+                # first pass: one launch per rank, the kernel's own barriers; second pass: a barrier launch either side
                 out = world.two_shot_all_reduce(t, own_barriers=(round_ == 0))
                 world.check()
                 save(directory, f"two_shot_{tag}.{round_}.out", rank, out)

@@ -87,31 +87,35 @@ def test_argument_checks_return_codes_without_launching():
     pads = _lib.ptr_array([0x5000, 0x6000])
     sz = lib.tccl_double_tree_signal_pad_bytes
     ctl = 288 * 4                                        # control words at the end of a pad
-    assert sz(8, 134_217_728, 0, 65_536) == 65_536 + ctl       # 2 trees x 1,024 chunks x 8 flags
-    assert sz(8, 134_217_728, 0, 0) == 262_144 + ctl           # default: 32 KiB chunks, 4,096 per tree
-    assert sz(8, 134_217_728, 0, 65_536 * 2) == 32_768 + ctl   # 512 chunks per tree
-    assert sz(2, 16, 0, 0) == 16 + ctl                         # one chunk per tree, two flags each
-    assert sz(2, 8, 1, 0) == 16 + ctl
+
+    def rows(world):                                     # two rows of barrier slots for 512 workgroups per rank
+        return 2 * 512 * world * 4
+
+    assert sz(8, 134_217_728, 0, 65_536) == 65_536 + rows(8) + ctl       # 2 trees x 1,024 chunks x 8 flags
+    assert sz(8, 134_217_728, 0, 0) == 262_144 + rows(8) + ctl           # default: 32 KiB chunks, 4,096 per tree
+    assert sz(8, 134_217_728, 0, 65_536 * 2) == 32_768 + rows(8) + ctl   # 512 chunks per tree
+    assert sz(2, 16, 0, 0) == 16 + rows(2) + ctl                         # one chunk per tree, two flags each
+    assert sz(2, 8, 1, 0) == 16 + rows(2) + ctl
     assert sz(3, 64, 0, 0) == 0 and sz(16, 64, 0, 0) == 0 and sz(8, 60, 0, 0) == 0 and sz(8, 64, 9, 0) == 0
     piped = lib.tccl_double_tree_all_reduce_pipelined
-    assert piped(good, None, pads, 4096, 3, 64, 0, 0, None, None) == -3
-    assert piped(good, None, pads, 4096, 16, 64, 0, 0, None, None) == -1
-    assert piped(good, None, pads, 4096, 2, 60, 0, 0, None, None) == -2
-    assert piped(good, None, pads, 4096, 2, 64, 0, 12, None, None) == -2      # chunk not whole vectors
-    assert piped(good, None, None, 4096, 2, 64, 0, 0, None, None) == -1
+    assert piped(good, None, pads, 16384, 3, 64, 0, 0, None, None) == -3
+    assert piped(good, None, pads, 16384, 16, 64, 0, 0, None, None) == -1
+    assert piped(good, None, pads, 16384, 2, 60, 0, 0, None, None) == -2
+    assert piped(good, None, pads, 16384, 2, 64, 0, 12, None, None) == -2      # chunk not whole vectors
+    assert piped(good, None, None, 16384, 2, 64, 0, 0, None, None) == -1
     assert piped(good, None, pads, 0, 2, 64, 0, 0, None, None) == -1          # pads too small
-    assert piped(null, None, pads, 4096, 2, 64, 0, 0, None, None) == -1
-    assert piped(odd, None, pads, 4096, 2, 64, 0, 0, None, None) == -2
-    assert piped(good, None, pads, 4096, 2, 0, 0, 0, None, None) == 0
+    assert piped(null, None, pads, 16384, 2, 64, 0, 0, None, None) == -1
+    assert piped(odd, None, pads, 16384, 2, 64, 0, 0, None, None) == -2
+    assert piped(good, None, pads, 16384, 2, 0, 0, 0, None, None) == 0
     ranked = lib.tccl_double_tree_all_reduce_pipelined_rank
-    assert ranked(good, None, pads, 4096, 2, 2, 64, 0, 0, None, None) == -1   # rank outside the world
-    assert ranked(good, None, pads, 4096, 2, -1, 64, 0, 0, None, None) == -1
-    assert ranked(good, None, pads, 4096, 3, 1, 64, 0, 0, None, None) == -3
-    assert ranked(good, None, pads, 4096, 2, 1, 60, 0, 0, None, None) == -2
+    assert ranked(good, None, pads, 16384, 2, 2, 64, 0, 0, None, None) == -1   # rank outside the world
+    assert ranked(good, None, pads, 16384, 2, -1, 64, 0, 0, None, None) == -1
+    assert ranked(good, None, pads, 16384, 3, 1, 64, 0, 0, None, None) == -3
+    assert ranked(good, None, pads, 16384, 2, 1, 60, 0, 0, None, None) == -2
     assert ranked(good, None, pads, 0, 2, 1, 64, 0, 0, None, None) == -1
     drawn = _lib.PipelineCfg(flags=_lib.PIPE_DRAW_PLACES)
-    assert ranked(good, None, pads, 4096, 2, 1, 64, 0, 0, ctypes.byref(drawn), None) == -1   # no drawn places per rank
-    assert ranked(good, None, pads, 4096, 2, 1, 0, 0, 0, None, None) == 0
+    assert ranked(good, None, pads, 16384, 2, 1, 64, 0, 0, ctypes.byref(drawn), None) == -1   # no drawn places per rank
+    assert ranked(good, None, pads, 16384, 2, 1, 0, 0, 0, None, None) == 0
     two = lib.tccl_two_shot_all_reduce
     assert two(good, None, pads, 4096, 0, 64, 0, None, None) == -1
     assert two(good, None, pads, 4096, 9, 64, 0, None, None) == -1
@@ -245,3 +249,54 @@ def test_struct_layouts_match_the_header(tmp_path):
                     P.timeout_flag.offset, P.flags.offset]
     assert consts == [_lib.ABI_VERSION, _lib.MAX_WORLD, _lib.MAX_JOBS, _lib.TCCL_BF16, _lib.TCCL_F32,
                       _lib.CFG_PHASED]
+
+
+def test_stamped_build_exports_the_same_abi_plus_its_stamp_buffer():
+    """benchlib/libtccl_amd_stamped.so is the library's own sources compiled with time stamps (for
+    ``bench.py --only OP --stamps``): it must export every entry point of the product, so that an
+    operation runs through the same wrappers, and the product must know nothing of the stamps."""
+    path = os.path.join(ROOT, "benchlib", "libtccl_amd_stamped.so")
+    assert os.path.exists(path), "run python -m tccl_amd.build"
+    stamped = ctypes.CDLL(path)
+    for name in _lib.SIGNATURES:
+        assert hasattr(stamped, name), f"{name} is missing from the stamped build"
+    assert hasattr(stamped, "tccl_stamp_buffer")
+    assert not hasattr(tccl_amd.load_library(), "tccl_stamp_buffer")
+    stamped.tccl_stamp_buffer.restype = ctypes.c_int
+    assert stamped.tccl_stamp_buffer(None, None, None) == _lib.TCCL_EINVAL
+
+
+def test_per_rank_entry_points_check_their_arguments():
+    """The one-shot collectives as one rank's launch: every refusal comes before anything is launched."""
+    lib = tccl_amd.load_library()
+    bufs = _lib.ptr_array([0x1000, 0x2000])
+    pads = _lib.ptr_array([0x5000, 0x6000])
+    big = 4 * (2 * 2 + 288)
+    out = ctypes.c_void_p(0x3000)
+    # (a launch needs a GPU: nothing here is called with arguments that would pass)
+    ar, rs, ag = lib.tccl_all_reduce_sum_rank, lib.tccl_reduce_scatter_sum_rank, lib.tccl_all_gather_rank
+    assert ar(None, out, pads, big, 2, 0, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL
+    assert ar(bufs, None, pads, big, 2, 0, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL
+    assert ar(bufs, out, None, big, 2, 0, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL
+    assert ar(bufs, out, pads, big, 2, 2, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL          # rank outside the world
+    assert ar(bufs, out, pads, big, 9, 0, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL
+    assert ar(bufs, out, pads, big - 16, 2, 0, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL     # no room for two rows of slots
+    assert ar(bufs, out, pads, big, 2, 0, 64, 7, None, None) == _lib.TCCL_EINVAL                       # unknown dtype
+    assert ar(bufs, out, pads, big, 2, 0, 60, _lib.TCCL_BF16, None, None) == _lib.TCCL_EALIGN          # not whole vectors
+    assert ar(_lib.ptr_array([0x1000, 0x2008]), out, pads, big, 2, 0, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EALIGN
+    assert ar(bufs, out, _lib.ptr_array([0x5000, 0x6004]), big, 2, 0, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EALIGN
+    drawn = _lib.PipelineCfg()
+    drawn.flags = _lib.PIPE_DRAW_PLACES
+    assert ar(bufs, out, pads, big, 2, 0, 64, _lib.TCCL_BF16, ctypes.byref(drawn), None) == _lib.TCCL_EINVAL
+    assert rs(bufs, out, pads, big, 2, 0, 72, _lib.TCCL_BF16, None, None) == _lib.TCCL_EALIGN          # shares would be ragged
+    assert rs(bufs, out, pads, big, 2, 0, 65, _lib.TCCL_BF16, None, None) == _lib.TCCL_EALIGN
+    assert rs(bufs, out, pads, big, 2, 3, 64, _lib.TCCL_BF16, None, None) == _lib.TCCL_EINVAL
+    assert ag(bufs, out, pads, big, 2, 0, 24, None, None) == _lib.TCCL_EALIGN
+    assert ag(bufs, None, pads, big, 2, 0, 32, None, None) == _lib.TCCL_EINVAL
+    # the two-shot and double-tree launches of one rank with their own barriers need more rows of slots
+    own = _lib.PipelineCfg()
+    own.flags = _lib.PIPE_OWN_BARRIERS
+    small = 4 * (2 + 288)
+    ts = lib.tccl_two_shot_all_reduce_rank
+    assert ts(bufs, None, pads, small, 2, 0, 64, _lib.TCCL_BF16, ctypes.byref(own), None) == _lib.TCCL_EINVAL
+    assert lib.tccl_double_tree_signal_pad_bytes(8, 1 << 20, _lib.TCCL_BF16, 0) >= 4 * (2 * 512 * 8 + 288)

@@ -52,3 +52,20 @@ def test_sweep_runs_and_prints_the_reference_columns(op, tmp_path):
     if op in ("double_tree_pipelined", "two_shot_world"):
         assert "expired waits: 0" in proc.stdout
     assert png.exists() and png.read_bytes()[:4] == b"\x89PNG"
+
+
+@pytest.mark.gpu
+def test_bench_prints_a_stamp_table_for_one_operation():
+    """``python bench.py --only c1 --stamps``: the measurement build of the library (every kernel with
+    per-workgroup time stamps) loads, runs the operation through the same entry points, and the table
+    it prints holds the 512 workgroups of the W=8 x 8 MiB launch with times that make sense."""
+    cmd = [sys.executable, os.path.join(ROOT, "bench.py"), "--only", "c1", "--stamps", "--steps", "3", "--warmup", "8"]
+    proc = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=150)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    out = proc.stdout
+    assert "512 workgroups stamped" in out and "last store acked" in out
+    rows = [ln.split() for ln in out.splitlines() if ln.startswith("all ")]
+    assert len(rows) == 1
+    numbers = [float(v) for v in rows[0] if v.replace(".", "").isdigit()]
+    start_max, first_data, last_load, last_store = numbers[1], numbers[2], numbers[4], numbers[7]
+    assert start_max < first_data < last_load < last_store < 100.0          # microseconds after the first workgroup started
