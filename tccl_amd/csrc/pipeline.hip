@@ -1110,7 +1110,9 @@ __device__ __forceinline__ bool rank_barrier(const RankArgs &a, uint32_t row, in
 }
 
 // 16 KiB tiles, as in the two-shot kernel: a rank has 1/W of the GPU's workgroup slots, and
-// small tiles spread a small input over all of them.
+// small tiles spread a small input over all of them.  (Tiles of 32, 64 and 128 KiB measured within
+// 10 % of these either way at 1 to 256 MiB per buffer with 8 processes, which is the spread between
+// two runs.)
 constexpr int kRankVecs = 4;
 
 // All-reduce (bytes = the whole buffer) and reduce-scatter (src offset to this rank's share,
