@@ -11,6 +11,12 @@ with HIP events on the launch stream.
     python -m tccl_amd.harness all_reduce|reduce_scatter|all_gather|double_tree|double_tree_pipelined|
                                two_shot|two_shot_world [--world 8] [--max-elems N] [--compare] [--plot out.png]
 
+Started once per rank (``python -m tccl_amd.launch --nproc-per-node 8 --module tccl_amd.harness all_reduce``) it is the
+reference's benchmark as the reference runs it: every rank a process of its own with its own symmetric
+buffer (``tccl_amd.ipc.IpcWorld``), every call one launch per rank with the blockwise barrier inside,
+rank 0 printing the lines; the operations are then ``all_reduce``, ``reduce_scatter``, ``all_gather``,
+``two_shot``, ``double_tree`` and ``auto`` (``tccl_amd.all_reduce(tensor)``: the algorithm picked by size).
+
 ``--plot`` draws what the reference's notebook draws (plot.ipynb: message size against rate, both
 axes logarithmic, one curve per implementation) from the lines just printed, with the axis in
 GB/s as measured (the notebook multiplies its GB/s by 1e6 and calls them B/s).
@@ -19,6 +25,7 @@ from __future__ import annotations
 
 import argparse
 import ctypes
+import os
 import sys
 
 import re
@@ -63,10 +70,70 @@ def plot(lines: List[str], path: str, title: str) -> None:
     plt.close(fig)
 
 
+def per_rank_main(args) -> int:
+    """This process is one rank (started by ``python -m tccl_amd.launch``): the reference's benchmark loop
+    (triton_reduce_scatter.py:213-240) on this rank's symmetric buffer, the peers being other processes."""
+    import torch
+    import tccl_amd
+    from tccl_amd import ipc
+    world = ipc.IpcWorld.from_env()
+    rank, size = world.rank, world.world_size
+    ops = {
+        "all_reduce": (tccl_amd.one_shot_all_reduce, lambda n: (size + 1) * n * 2),
+        "reduce_scatter": (tccl_amd.reduce_scatter, lambda n: (size + 1) * (n // size) * 2),
+        "all_gather": (lambda t: tccl_amd.all_gather(t, size), lambda n: 2 * size * n * 2),
+        "two_shot": (tccl_amd.two_shot_all_reduce, lambda n: (3 * size - 1) * (n // size) * 2),
+        "double_tree": (tccl_amd.double_tree_all_reduce, None),
+        "auto": (tccl_amd.all_reduce, None),
+    }
+    if args.op not in ops:
+        if rank == 0:
+            print(f"{args.op} runs every rank's work from one process; with a process per rank use one of {sorted(ops)}",
+                  file=sys.stderr)
+        world.close()
+        return 2
+    fn, algo_bytes = ops[args.op]
+    max_elems = args.max_elems // (8 * size) * (8 * size)
+    tensor = world.empty(max_elems, torch.bfloat16)
+    torch.manual_seed(rank)
+    tensor.copy_(torch.randn(1 << 16, dtype=torch.bfloat16).repeat(-(-max_elems // (1 << 16)))[:max_elems] * (1.0 / 64))
+    in_place = args.op in ("two_shot", "double_tree", "auto")
+    printed: List[str] = []
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n = max_elems
+    while n >= 2048:
+        n = n // (8 * size) * (8 * size)
+        view = tensor[:n]
+        fn(view)                                    # warm-up (the reference has none)
+        start.record()
+        for _ in range(REPS):
+            if in_place:
+                view.mul_(1.0 / size)               # an in-place sum over and over would run away; part of the time
+            fn(view)
+        stop.record()
+        stop.synchronize()
+        world.check()
+        per_call_ms = start.elapsed_time(stop) / REPS
+        if rank == 0:
+            line = f"tccl_amd {n * 2} {n * 2 / per_call_ms / 1e6:.3f} GB/s"
+            if algo_bytes is not None:
+                line += f"  (HBM {algo_bytes(n) / per_call_ms / 1e6:.1f} GB/s for this rank, {per_call_ms * 1e3:.1f} us)"
+            else:
+                line += f"  ({per_call_ms * 1e3:.1f} us" + (f", {world.auto_algorithm(view)})" if args.op == "auto" else ")")
+            printed.append(line)
+            print(line, flush=True)
+        n //= 2
+    world.close()
+    if rank == 0 and args.plot:
+        plot(printed, args.plot, f"{args.op}, {size} processes (one rank each) on one MI355X")
+        print(f"plot written to {args.plot}", flush=True)
+    return 0
+
+
 def main(argv=None) -> int:
     p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     p.add_argument("op", choices=["all_reduce", "reduce_scatter", "all_gather", "double_tree", "double_tree_plan", "double_tree_fused",
-                                  "double_tree_pipelined", "two_shot", "two_shot_world"])
+                                  "double_tree_pipelined", "two_shot", "two_shot_world", "auto"])
     p.add_argument("--world", type=int, default=8)
     p.add_argument("--max-elems", type=int, default=256 * 1024 * 1024 // 2,
                    help="largest element count per rank (bf16); halved down to 2,048")
@@ -75,6 +142,10 @@ def main(argv=None) -> int:
                    help="also time the same operation written with torch's own GPU kernels, as the second "
                         "line per size (the place the reference gives to NCCL)")
     args = p.parse_args(argv)
+    if "RANK" in os.environ and "TCCL_RENDEZVOUS_DIR" in os.environ:
+        return per_rank_main(args)
+    if args.op == "auto":
+        p.error("auto is an operation of the per-rank form (start the harness through python -m tccl_amd.launch)")
 
     import torch
     import tccl_amd

@@ -69,3 +69,18 @@ def test_bench_prints_a_stamp_table_for_one_operation():
     numbers = [float(v) for v in rows[0] if v.replace(".", "").isdigit()]
     start_max, first_data, last_load, last_store = numbers[1], numbers[2], numbers[4], numbers[7]
     assert start_max < first_data < last_load < last_store < 100.0          # microseconds after the first workgroup started
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("op", ["all_reduce", "reduce_scatter", "all_gather", "two_shot", "double_tree", "auto"])
+def test_sweep_with_a_process_per_rank(op):
+    """The same sweep started once per rank, as the reference's benchmarks are started by torchrun: 4 processes,
+    every call one launch per rank; rank 0 prints the reference's columns."""
+    cmd = [sys.executable, "-m", "tccl_amd.launch", "--nproc-per-node", "4", "--module", "tccl_amd.harness", op,
+           "--max-elems", str(1 << 20)]
+    proc = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=150)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    recs = [harness.parse_line(ln) for ln in proc.stdout.splitlines()]
+    recs = [r for r in recs if r is not None]
+    assert [r[1] for r in recs] == [2 * ((1 << 20) >> i) for i in range(10)], proc.stdout
+    assert all(r[0] == "tccl_amd" and 0 < r[2] < float("inf") for r in recs)
