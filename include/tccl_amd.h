@@ -314,7 +314,10 @@ int tccl_two_shot_all_reduce(void *const *bufs, void *const *outs, void *const *
  * With TCCL_PIPE_OWN_BARRIERS in cfg->flags the kernel also begins and ends with that barrier, as
  * the reference's kernels begin with it (triton_one_shot_all_reduce_no_128.py:46), and no
  * tccl_blockwise_barrier() before or after is needed: one launch per rank per collective.  The pads
- * then hold three rows of slots per workgroup, pad_bytes >= 4 * (3 * world + TCCL_PAD_CONTROL_WORDS).
+ * then hold three rows of slots per workgroup, pad_bytes >= 4 * (3 * world + TCCL_PAD_CONTROL_WORDS);
+ * calls that follow each other without a host-side meeting of the ranks in between must be given
+ * the same pad_bytes and world, which fix where a workgroup's rows lie, and pads of their own (not
+ * those of the one-shot or double-tree entry points).
  * An empty input launches nothing and orders nothing. */
 int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void *const *signal_pads,
                                   size_t pad_bytes, int world, int rank, size_t numel, int dtype,
@@ -343,7 +346,9 @@ int tccl_two_shot_all_reduce_rank(void *const *bufs, void *out, void *const *sig
  * call, pad_bytes >= 4 * (2 * world + TCCL_PAD_CONTROL_WORDS) (two rows of slots per workgroup:
  * the leading and the trailing barrier alternate between them, so a flag is never raised over
  * one that has not been consumed); larger pads allow more workgroups per rank.  The same pads
- * may serve any sequence of these three calls.  Waits are bounded (cfg->spin_limit, cfg->timeout_flag, the
+ * may serve any sequence of these three calls, of any sizes, as long as every call is given the
+ * same pad_bytes and world (they fix where a workgroup's two rows lie); they may not be shared
+ * with the two-shot or double-tree entry points, which lay their rows out differently.  Waits are bounded (cfg->spin_limit, cfg->timeout_flag, the
  * time-out count in the last word of pad 0): a rank whose peers do not arrive gives up, leaves
  * `out` unwritten or partly written, and says so.  TCCL_PIPE_DRAW_PLACES does not apply
  * (TCCL_EINVAL); cfg->lag and cfg->tile_kib are unused.  Preconditions on the sizes as for the
@@ -389,7 +394,7 @@ int tccl_timeout_flag_destroy(uint32_t *flag);
 /* Buffers that several processes on one GPU can map: what the reference gets from
  * _SymmetricMemory.empty_strided_p2p (triton_one_shot_all_reduce_no_128.py:116-122) and
  * rendezvous (:82).  tccl_symm_alloc returns a zero-filled device allocation of its own (below
- * 2 GiB); tccl_ipc_export writes its 64-byte handle, which the host side carries to the peers;
+ * 2 GiB; it waits for the null stream, so the zeros are in place before a peer can map it); tccl_ipc_export writes its 64-byte handle, which the host side carries to the peers;
  * tccl_ipc_open maps a peer's allocation into this process and returns its address here, good for
  * every pointer table of this header; tccl_ipc_close unmaps it.  These four calls allocate, map or
  * synchronise: they belong to set-up, not to the hot path. */

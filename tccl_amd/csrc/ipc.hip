@@ -87,7 +87,12 @@ extern "C" int tccl_symm_alloc(size_t bytes, void **ptr_out)
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, bytes);
     if (e != hipSuccess) return hip_code(e);
+    // hipMemset on device memory may return before the fill has run (it is queued on the null
+    // stream, behind whatever this process has in flight there).  The caller exports the
+    // allocation next, and a peer that maps it may raise flags in it straight away: the zeros
+    // must be in place before this call returns, or the late fill would wipe those flags out.
     e = hipMemset(p, 0, bytes);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
     if (e != hipSuccess) {
         (void)hipFree(p);
         return hip_code(e);

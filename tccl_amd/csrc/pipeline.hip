@@ -436,7 +436,7 @@ __device__ __forceinline__ void tree_pipelined_walk(const PipeArgs &a, int rank,
     if (g >= most) return; // (the same workgroups in every rank's launch)
     // One launch per rank with the reference's leading barrier inside (the double tree's kernel
     // begins with blockwise_barrier, triton_double_tree_allreduce.py:239): every rank's input is
-    // in place before anybody reads a leaf's buffer.  The trailing barrier (row G + g) tells the
+    // in place before anybody reads a leaf's buffer.  The trailing barrier (row 512 + g) tells the
     // peers that this workgroup has taken every flag and read every chunk it ever will, so buffers
     // and pads are free for the next collective when the kernel has ended.  Two rows in turn, as
     // in the one-shot kernels.
@@ -464,7 +464,9 @@ __device__ __forceinline__ void tree_pipelined_walk(const PipeArgs &a, int rank,
     if (own_barriers) {
         __syncthreads();
         if (threadIdx.x == 0) *lds_ok = 1;
-        (void)barrier_on_slots(a.pad, a.world, rank, a.barrier_base + (G + g) * a.world, a.spin_limit, a.ctl, a.report, lds_ok);
+        // (the second block of rows starts at a fixed row, not at G: calls with different G share the pads)
+        const uint32_t row = static_cast<uint32_t>(kTreeBarrierWorkgroups) + g;
+        (void)barrier_on_slots(a.pad, a.world, rank, a.barrier_base + row * a.world, a.spin_limit, a.ctl, a.report, lds_ok);
     }
 }
 
@@ -788,6 +790,7 @@ struct TwoShotArgs {
     int draw;         // 1 = workgroups draw their places when they start, 0 = places follow the hardware index
     int only_rank;    // >= 0: the launch holds this rank's workgroups only (one launch per rank); -1: all ranks'
     int own_barriers; // one launch per rank: the kernel also begins and ends with the blockwise barrier
+    uint32_t rows;    // own_barriers: rows of one barrier's block of the pad (fixed by the pad's size, not by G)
     uint32_t *ctl;    // control words at the end of pad 0 (place counters ... time-outs)
     uint32_t *report; // optional host word set to 1 when a wait expires
 };
@@ -814,10 +817,13 @@ constexpr int kTwoShotVecs = 4;
 //
 // PEERS_MAY_STILL_WRITE (one launch per rank): the kernel may have started before a peer's
 // producer kernel ended, so shot 1 reads with device-scope loads too; and with a.own_barriers
-// the kernel begins with the barrier that says "every rank's input is in place" (row G + g of
+// the kernel begins with the barrier that says "every rank's input is in place" (row R + g of
 // the pads) and ends with the one that says "every rank has read what it needs from every
-// buffer" (row 2 G + g) -- three barriers in a row on three different rows, so a flag is never
-// raised over one that its reader has not consumed, within a call and from call to call.
+// buffer" (row 2 R + g) -- three barriers in a row on three different rows, so a flag is never
+// raised over one that its reader has not consumed, within a call and from call to call.  R is
+// a third of the pad's rows whatever G is: a call with more workgroups than the one before it
+// (a larger input) must find workgroup g's rows where the last call left them, or its leading
+// flags would land on trailing flags of the last call that a slower peer has yet to take.
 template <class Sum, int W, bool PEERS_MAY_STILL_WRITE>
 __device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, uint32_t g, int &lds_ok)
 {
@@ -831,7 +837,7 @@ __device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, ui
     if (threadIdx.x == 0) lds_ok = 1;
     // (the barrier's first __syncthreads orders this store before any lane's clear)
     const bool own_barriers = PEERS_MAY_STILL_WRITE && W > 1 && a.own_barriers != 0;
-    if (own_barriers && !blockwise_barrier(a, rank, G + g, &lds_ok)) return;
+    if (own_barriers && !blockwise_barrier(a, rank, a.rows + g, &lds_ok)) return;
 
     const char *src[W];
 #pragma unroll
@@ -878,7 +884,7 @@ __device__ __forceinline__ void two_shot_body(const TwoShotArgs &a, int rank, ui
             }
         }
     }
-    if (own_barriers) (void)blockwise_barrier(a, rank, 2 * G + g, &lds_ok);
+    if (own_barriers) (void)blockwise_barrier(a, rank, 2 * a.rows + g, &lds_ok);
 }
 
 template <class Sum, int W>
@@ -940,6 +946,7 @@ static int launch_two_shot(TwoShotArgs a, int wgs_wanted, size_t pad_words, cons
     // trailing barriers; the last words of pad 0 are the control words
     const size_t fit = (pad_words - kCtlWords) / (static_cast<size_t>(W) * (a.own_barriers ? 3 : 1));
     if (fit < 1) return TCCL_EINVAL;
+    a.rows = static_cast<uint32_t>(fit);
     size_t per_rank;
     if (wgs_wanted > 0) {
         per_rank = static_cast<size_t>((wgs_wanted < resident ? wgs_wanted : resident) / W);
@@ -1086,7 +1093,12 @@ namespace tccl {
 // plus the barrier the reference lacks at the end ("I have read your buffer, refill it").
 //
 // The two barriers of a call use different rows of slots: row g for the leading one, row
-// wgs + g for the trailing one.  A rank raises its flag for barrier k+1 of a row only after
+// R + g for the trailing one, R = half the rows the pad holds -- fixed by the pad, not by the
+// launch, so that workgroup g finds its rows in the same place in every call on the same pads
+// whatever the calls' sizes and kinds.  (With R = this launch's workgroup count, a call with
+// more workgroups than the one before it would raise leading flags on rows where a slower
+// peer has yet to take the last call's trailing flags, and one of the two would be lost.)
+// A rank raises its flag for barrier k+1 of a row only after
 // it has passed barrier k of the other row, which its peer raises only after it has lowered
 // the flag of barrier k of this row -- so a flag is never raised over one that has not been
 // consumed, within a call and from call to call, without the sender having to wait for the
@@ -1098,6 +1110,7 @@ struct RankArgs {
     size_t bytes; // sums: bytes to reduce; gather: bytes per rank
     uint32_t spin_limit;
     int world, rank, wgs;
+    uint32_t rows;    // R: the trailing barrier's first row
     uint32_t *ctl;    // control words at the end of pad 0 (time-outs)
     uint32_t *report; // optional host word set to 1 when a wait expires
 };
@@ -1146,7 +1159,7 @@ __global__ void __launch_bounds__(kPhasedBlock) sum_rank_kernel(RankArgs a)
             sum_tile_phased<Sum, W, 1, U, KMAX, false, false, kAuxLoadDevice>(csrc, dst, t, valid,
                                                                               static_cast<int>((valid + span - 1) / span));
     }
-    if (W > 1) (void)rank_barrier(a, G + g, &lds_ok);
+    if (W > 1) (void)rank_barrier(a, a.rows + g, &lds_ok);
 }
 
 // All-gather: out[s] = rank s's buffer for every s, starting at a different peer per rank.
@@ -1168,7 +1181,7 @@ __global__ void __launch_bounds__(kPhasedBlock) gather_rank_kernel(RankArgs a)
             copy_tile_phased<1, 4, VECS / 4, kAuxLoadDevice>(a.src[s], dst, t, valid, static_cast<int>((valid + span - 1) / span));
         }
     }
-    if (a.world > 1) (void)rank_barrier(a, G + g, &lds_ok);
+    if (a.world > 1) (void)rank_barrier(a, a.rows + g, &lds_ok);
 }
 
 // Every rank computes the same count from the same arguments: its launch takes 1/W of the
@@ -1181,6 +1194,7 @@ static int launch_rank_kernel(K kernel, int resident, RankArgs a, size_t tiles, 
     // two rows of slots (leading and trailing barrier), one slot per (workgroup, sender)
     const size_t fit = (pad_words - kCtlWords) / (2 * static_cast<size_t>(a.world));
     if (fit < 1) return TCCL_EINVAL;
+    a.rows = static_cast<uint32_t>(fit);
     size_t most = static_cast<size_t>(resident / a.world);
     if (most > fit) most = fit;
     size_t per_rank;

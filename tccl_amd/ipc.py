@@ -8,16 +8,22 @@ for W processes that share one MI355X: a rank's buffer is a device allocation of
 they all see, and mapped there (``tccl_ipc_open``).  The resulting ``SymmHandle`` goes through
 the same wrappers as a group of virtual ranks (``one_shot_all_reduce``, ``reduce_scatter``,
 ``all_gather``); ordering between the ranks' launches is the reference's device-side
-``blockwise_barrier`` (triton_barrier.py:39-142), one kernel launch per rank
-(``IpcWorld.barrier``), before a collective and -- what the reference lacks -- after it.
+``blockwise_barrier`` (triton_barrier.py:39-142) inside the collective's kernel, as the reference
+has it (triton_one_shot_all_reduce_no_128.py:46), before the first read and -- what the reference
+lacks -- after the last one: a collective is one launch per rank, and when it has ended on a
+rank's stream that rank may refill its buffer.  (Large one-shot inputs run as barrier launch, the
+full-size kernel, barrier launch instead: ``IpcWorld.FUSED_MAX_MOVED_BYTES``.)
 
     world = IpcWorld(rank, world_size, directory)          # one per process
     tensor = world.empty(numel, torch.bfloat16)            # this rank's buffer, peers mapped
     tensor.copy_(...)
-    world.barrier()                                        # every rank's buffer is filled
-    out = tccl_amd.one_shot_all_reduce(tensor)
-    world.barrier()                                        # every rank has read it
+    out = tccl_amd.one_shot_all_reduce(tensor)             # waits for the peers' buffers itself
+    world.check()                                          # raises if a wait inside a kernel expired
     world.close()
+
+``IpcWorld.barrier`` is the barrier alone (one launch per rank), ``IpcWorld.all_reduce`` picks
+between the one-shot, two-shot and double-tree forms by size, ``IpcWorld.reset`` clears the pads
+after a time-out.
 """
 from __future__ import annotations
 
@@ -79,7 +85,7 @@ class IpcWorld:
         self._allocs: List[int] = []          # own allocations
         self._opened: List[int] = []          # peers' allocations mapped here
         self._tables = {}                     # own buffer address -> (all ranks' addresses, bytes, dtype)
-        self._tree_pads = {}                  # pad size -> table of all ranks' pads for kernels that signal inside a launch
+        self._tree_pads = {}                  # (kernel family, pad size) -> table of all ranks' pads for kernels that signal inside a launch
         self._count = 0
         self._host_barriers = 0
         self._epoch = 0                       # resets so far: time-outs are published per epoch
@@ -90,7 +96,7 @@ class IpcWorld:
         self._pad_array = _lib.ptr_array(self._pad_ptrs)
         # ... and the pads of the one-shot kernels that carry their barriers themselves, so that a rank's
         # first collective never has to wait on the host for a peer that is late
-        self._kernel_pads(self.ONE_SHOT_PAD_BYTES)
+        self._kernel_pads(self.ONE_SHOT_PAD_BYTES, "one_shot")
 
     @classmethod
     def from_env(cls, device="cuda:0", timeout_s: float = 60.0) -> "IpcWorld":
@@ -200,18 +206,22 @@ class IpcWorld:
     # Signal pad size the two-shot kernel is given: room for 1024 workgroups per rank.
     TWO_SHOT_PAD_BYTES = 4 * (8 * 1024 + 288)
 
-    def _kernel_pads(self, nbytes: int) -> ctypes.Array:
-        """All ranks' signal pads of `nbytes` for the kernels that signal inside a launch (collective on
-        first use of a size, like ``empty``)."""
-        if nbytes not in self._tree_pads:
-            self._tree_pads[nbytes] = _lib.ptr_array(self._exchange(self._alloc(nbytes), "kpad"))
-        return self._tree_pads[nbytes]
+    def _kernel_pads(self, nbytes: int, family: str) -> ctypes.Array:
+        """All ranks' signal pads of `nbytes` for the kernels of one family ("one_shot", "two_shot",
+        "double_tree") that signal inside a launch (collective on first use, like ``empty``).  Every
+        family has pads of its own: each lays its barrier rows out differently, and a kernel that ends
+        while a slower peer has yet to take its last flags may only be followed, on the same pads, by a
+        kernel that keeps those rows for the same purpose."""
+        key = (family, nbytes)
+        if key not in self._tree_pads:
+            self._tree_pads[key] = _lib.ptr_array(self._exchange(self._alloc(nbytes), "kpad"))
+        return self._tree_pads[key]
 
-    def _own_launch(self, name: str, tensor: torch.Tensor, pad_bytes: int, tail_args, cfg,
+    def _own_launch(self, name: str, family: str, tensor: torch.Tensor, pad_bytes: int, tail_args, cfg,
                     own_barriers: bool = False) -> torch.Tensor:
         ptrs, _, dtype = self._tables[self._base(tensor)]
         code = {torch.bfloat16: _lib.TCCL_BF16, torch.float32: _lib.TCCL_F32}[dtype]
-        pads = self._kernel_pads(pad_bytes)
+        pads = self._kernel_pads(pad_bytes, family)
         use = _lib.PipelineCfg()
         if cfg is not None:
             ctypes.memmove(ctypes.byref(use), ctypes.byref(cfg), ctypes.sizeof(use))
@@ -244,7 +254,7 @@ class IpcWorld:
             raise ValueError("the pipelined double tree takes worlds of 2, 4 or 8 and whole 16-byte vectors")
         if tensor.numel() == 0:
             return torch.empty_like(tensor)
-        return self._own_launch("tccl_double_tree_all_reduce_pipelined_rank", tensor, need, (chunk_elems,), cfg, own_barriers)
+        return self._own_launch("tccl_double_tree_all_reduce_pipelined_rank", "double_tree", tensor, need, (chunk_elems,), cfg, own_barriers)
 
     def two_shot_all_reduce(self, tensor: torch.Tensor, cfg: Optional[_lib.PipelineCfg] = None,
                             own_barriers: bool = True) -> torch.Tensor:
@@ -257,7 +267,7 @@ class IpcWorld:
         False = a barrier launch before and after instead."""
         if tensor.numel() == 0:
             return torch.empty_like(tensor)
-        return self._own_launch("tccl_two_shot_all_reduce_rank", tensor, self.TWO_SHOT_PAD_BYTES, (), cfg, own_barriers)
+        return self._own_launch("tccl_two_shot_all_reduce_rank", "two_shot", tensor, self.TWO_SHOT_PAD_BYTES, (), cfg, own_barriers)
 
     # Signal pad size of the one-shot kernels: two rows of slots for up to 512 workgroups per rank.
     ONE_SHOT_PAD_BYTES = 4 * (2 * 8 * 512 + 288)
@@ -291,7 +301,7 @@ class IpcWorld:
             _lib.check(plain, getattr(self.lib, plain)(*args, stream))
             self.barrier()                                     # every rank has read every buffer
             return out
-        pads = self._kernel_pads(self.ONE_SHOT_PAD_BYTES)
+        pads = self._kernel_pads(self.ONE_SHOT_PAD_BYTES, "one_shot")
         use = _lib.PipelineCfg()
         if cfg is not None:
             ctypes.memmove(ctypes.byref(use), ctypes.byref(cfg), ctypes.sizeof(use))
@@ -417,7 +427,7 @@ class IpcWorld:
         _as_tensor(self._pad_ptrs[self.rank], self.PAD_BYTES, self.device).zero_()
         # the pads of the kernels that signal inside a launch, control words included: a wait that
         # expired there leaves flags standing that the next collective would take for its own
-        for nbytes, table in self._tree_pads.items():
+        for (_, nbytes), table in self._tree_pads.items():
             _as_tensor(table[self.rank], nbytes, self.device).zero_()
         torch.cuda.synchronize(self.device)
         self._flag[0] = 0

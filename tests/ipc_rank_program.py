@@ -34,6 +34,12 @@ ONE_SHOT_SHAPES = (("small", 8 * 5, torch.bfloat16), ("ragged", 8 * 4099, torch.
                    ("big", 8 * 131_072, torch.bfloat16))
 
 
+# elements per rank's share of the three buffer sizes of the mixed sequence: one workgroup per rank,
+# a few dozen, and every workgroup a rank's launch may hold
+MIXED_SHARES = (("tiny", 8 * 3), ("mid", 8 * 4099), ("big", 8 * 131_072))
+MIXED_ROUNDS = 4
+
+
 def AUTO_SIZES(world_size, edge):
     """(name, bf16 elements): small; at the threshold of "auto"; one step (W vectors) above it; a buffer
     large enough that a one-shot all-reduce is three launches again."""
@@ -97,7 +103,7 @@ def main():
                     save(directory, f"rank_{name}_{tag}.{round_}", rank, o)
             world.check()
             print(f"rank {rank}: one-shot kernels {tag} done", flush=True)
-        pad = world._kernel_pads(world.ONE_SHOT_PAD_BYTES)
+        pad = world._kernel_pads(world.ONE_SHOT_PAD_BYTES, "one_shot")
         own = ipc._as_tensor(pad[rank], world.ONE_SHOT_PAD_BYTES, world.device).view(torch.int32)
         world.barrier()
         left = int(own.ne(0).sum())
@@ -106,6 +112,48 @@ def main():
         if left:
             print(f"rank {rank}: {left} words of the signal pad are not zero after the collectives", flush=True)
             return 5
+        return 0
+
+    if mode == "mixed_sequence":
+        # collectives of different kinds and very different sizes back to back, ranks out of step, no
+        # meeting on the host anywhere: a launch with many workgroups follows one with few on the same
+        # pads (and the other way round), one-shot, two-shot and double-tree kernels follow each other.
+        # Every kernel's flags must land where its peers' kernels of the SAME call look for them and
+        # nowhere else, whatever ran just before.
+        bufs = {tag: world.empty(share * world_size, torch.bfloat16) for tag, share in MIXED_SHARES}
+        inplace = {tag: world.empty(share * world_size, torch.bfloat16) for tag, share in MIXED_SHARES}
+        keep = {}
+        for tag, share in MIXED_SHARES:
+            fill(bufs[tag], share * world_size, torch.bfloat16, 700 + rank)
+            keep[tag] = bufs[tag].clone()
+        trees = world_size in (2, 4, 8)
+        results = []
+        for round_ in range(MIXED_ROUNDS):
+            if (round_ + rank) % 3 == 0:
+                torch.cuda._sleep(3_000_000)
+            order = ("tiny", "big", "mid", "big", "tiny") if round_ % 2 == 0 else ("big", "tiny", "mid", "tiny", "big")
+            for step, tag in enumerate(order):
+                kind = ("reduce_scatter", "all_reduce", "all_gather", "two_shot", "double_tree")[(step + round_) % 5]
+                if kind == "double_tree" and not trees:
+                    kind = "two_shot"
+                if kind == "reduce_scatter":
+                    out = world.reduce_scatter(bufs[tag], fused=True)
+                elif kind == "all_reduce":
+                    out = world.one_shot_all_reduce(bufs[tag], fused=True)
+                elif kind == "all_gather":
+                    out = world.all_gather(bufs[tag], fused=True)
+                else:                                                  # in place: refill first (the last call's trailing
+                    inplace[tag].copy_(keep[tag])                      # barrier has made that safe)
+                    out = (world.two_shot_all_reduce(inplace[tag]) if kind == "two_shot"
+                           else world.double_tree_all_reduce(inplace[tag]))
+                results.append((f"mixed_{round_}_{step}_{kind}_{tag}", out))
+        torch.cuda.synchronize()
+        world.check()
+        for name, out in results:
+            save(directory, name, rank, out)
+        if rank == 0:
+            print("SEQUENCE " + " ".join(name for name, _ in results), flush=True)
+        world.close()
         return 0
 
     if mode == "one_shot_missing_peer":
@@ -145,7 +193,7 @@ def main():
         if rank == 1:
             torch.cuda._sleep(400_000_000)                # about 0.2 s on the GPU, bounded
         ptrs = tccl_amd._lib.ptr_array(world._tables[t.data_ptr()][0])
-        pads = world._kernel_pads(world.TWO_SHOT_PAD_BYTES)
+        pads = world._kernel_pads(world.TWO_SHOT_PAD_BYTES, "two_shot")
         cfg.timeout_flag = world._flag
         import ctypes
         rc = world.lib.tccl_two_shot_all_reduce_rank(ptrs, None, pads, world.TWO_SHOT_PAD_BYTES, world_size, rank, numel, 0,

@@ -139,6 +139,41 @@ def test_one_shot_kernels_with_their_barriers_inside(world, tmp_path):
                 assert torch.equal(got, stacked), f"{tag} round {round_} rank {r}: all-gather"
 
 
+@pytest.mark.parametrize("world", [8, 3])
+def test_mixed_sequence_of_kinds_and_sizes_without_host_meetings(world, tmp_path):
+    """One-shot, two-shot and double-tree kernels of one workgroup per rank up to every workgroup a rank
+    may hold, back to back on the same pads with the ranks out of step and no host meeting: a call with
+    many workgroups right after one with few (whose trailing flags a slow peer may not have taken yet)
+    and kernels of different families after each other.  Every output against the oracle, bit for bit."""
+    from ipc_rank_program import MIXED_SHARES
+    print(f"ipc: mixed sequence, {world} processes", flush=True)
+    codes, outs = run_ranks(world, tmp_path, "mixed_sequence", timeout=150)
+    assert codes == [0] * world, "\n".join(outs)
+    names = [line for line in outs[0].splitlines() if line.startswith("SEQUENCE ")][0].split()[1:]
+    assert len(names) == 20 and {n.rsplit("_", 1)[1] for n in names} == {"tiny", "mid", "big"}
+    want, stacked, tree = {}, {}, {}
+    for tag, share in MIXED_SHARES:
+        bufs = seeded_randn(world, share * world, seed_base=700)
+        want[tag] = torch_ref.all_reduce(bufs).view(torch.int16)
+        stacked[tag] = torch.stack(bufs).view(torch.int16)
+        if world in (2, 4, 8):                  # the trees add in their own order
+            tree[tag] = torch_ref.double_tree_all_reduce(bufs)[0].view(torch.int16)
+    shares = dict(MIXED_SHARES)
+    for name in names:
+        kind, tag = name.split("_", 3)[3].rsplit("_", 1)
+        for r in range(world):
+            got = load(tmp_path, name, r, torch.bfloat16).view(torch.int16)
+            if kind == "reduce_scatter":
+                expect = want[tag][r * shares[tag]:(r + 1) * shares[tag]]
+            elif kind == "all_gather":
+                expect = stacked[tag]
+            elif kind == "double_tree":
+                expect = tree[tag]
+            else:
+                expect = want[tag]
+            assert torch.equal(got.reshape(expect.shape), expect), f"{name} rank {r}"
+
+
 def test_one_shot_kernel_with_a_missing_peer_gives_up_and_says_so(tmp_path):
     """Failure handling forced from the host: rank 0 launches its all-reduce with a small spin limit and
     no peer ever does.  The kernel ends by itself at its leading barrier, the rank is told, and after a
