@@ -189,11 +189,12 @@ def main():
         fill(t, numel, torch.bfloat16, rank)
         cfg = tccl_amd._lib.PipelineCfg()
         cfg.spin_limit = 3000 if rank != 1 else 0
+        # (the pads first: allocating them is a meeting of the ranks on the host and waits for the own stream)
+        pads = world._kernel_pads(world.TWO_SHOT_PAD_BYTES, "two_shot")
         world.barrier()
         if rank == 1:
             torch.cuda._sleep(400_000_000)                # about 0.2 s on the GPU, bounded
         ptrs = tccl_amd._lib.ptr_array(world._tables[t.data_ptr()][0])
-        pads = world._kernel_pads(world.TWO_SHOT_PAD_BYTES, "two_shot")
         cfg.timeout_flag = world._flag
         import ctypes
         rc = world.lib.tccl_two_shot_all_reduce_rank(ptrs, None, pads, world.TWO_SHOT_PAD_BYTES, world_size, rank, numel, 0,
