@@ -7,7 +7,10 @@ by torchrun (triton_one_shot_all_reduce_no_128.py:99-110 reads RANK, LOCAL_RANK 
 Every rank is a process of its own with RANK = 0 .. W-1, WORLD_SIZE = W, LOCAL_RANK = 0 (all ranks
 share the one GPU) and TCCL_RENDEZVOUS_DIR = a fresh directory through which the ranks exchange
 their buffer handles; ``tccl_amd.ipc.IpcWorld.from_env()`` in the program picks these up.  The
-launcher itself never touches the GPU.  Its exit code is the first non-zero exit code of a rank."""
+launcher itself never touches the GPU.  Its exit code is the exit code of the first rank that
+failed (124 if the time limit ended the run).  When a rank fails, its peers would wait for it in the
+next rendezvous or barrier until their own bounded waits expire: they get ``--grace`` seconds to
+end by themselves and are stopped then, and so is every rank still running at ``--timeout``."""
 from __future__ import annotations
 
 import argparse
@@ -16,12 +19,14 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import time
 
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="python -m tccl_amd.launch", description=__doc__.split("\n\n")[0])
     ap.add_argument("--nproc-per-node", type=int, required=True, help="ranks (processes) to start, 1..8")
     ap.add_argument("--timeout", type=float, default=600.0, help="seconds before ranks still running are stopped")
+    ap.add_argument("--grace", type=float, default=10.0, help="seconds the other ranks may run on after one has failed")
     ap.add_argument("--module", help="run this module once per rank (python -m MODULE) instead of a program file")
     ap.add_argument("program", nargs="?", help="the per-rank program (a Python file)")
     ap.add_argument("args", nargs=argparse.REMAINDER, help="its arguments")
@@ -42,13 +47,23 @@ def main(argv=None) -> int:
                        TCCL_RENDEZVOUS_DIR=directory)
             procs.append(subprocess.Popen(command, env=env))
         code = 0
-        for p in procs:
-            try:
-                rc = p.wait(timeout=ns.timeout)
-            except subprocess.TimeoutExpired:
-                rc = 124
-            if rc != 0 and code == 0:
-                code = rc
+        deadline = time.monotonic() + ns.timeout
+        running = list(procs)
+        while running:
+            for p in list(running):
+                rc = p.poll()
+                if rc is None:
+                    continue
+                running.remove(p)
+                if rc != 0 and code == 0:            # the first failure: the others' time is limited from now on
+                    code = rc
+                    deadline = min(deadline, time.monotonic() + ns.grace)
+            if running and time.monotonic() >= deadline:
+                if code == 0:
+                    code = 124
+                break                                # what still runs is stopped below
+            if running:
+                time.sleep(0.05)
         return code
     finally:
         for p in procs:                      # exactly the processes started here

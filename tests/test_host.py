@@ -102,6 +102,23 @@ def test_launcher_sets_the_environment_and_hands_on_exit_codes(tmp_path):
     assert subprocess.run(cmd[:4] + ["9", str(prog)], cwd=root, timeout=60, stderr=subprocess.DEVNULL).returncode == 2
 
 
+def test_launcher_stops_the_peers_of_a_failed_rank_and_keeps_its_time_limit(tmp_path):
+    """A rank that fails leaves peers that would wait for it: they are stopped after the grace period and the
+    launcher hands on the failed rank's code; ranks still running at the time limit are stopped with 124."""
+    import time
+    prog = tmp_path / "prog.py"
+    prog.write_text("import os, sys, time\n"
+                    "if os.environ['RANK'] == sys.argv[1]:\n"
+                    "    sys.exit(7)\n"
+                    "time.sleep(120)\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, "-m", "tccl_amd.launch", "--nproc-per-node", "3"]
+    t0 = time.monotonic()
+    assert subprocess.run(cmd + ["--grace", "1", str(prog), "1"], cwd=root, timeout=60).returncode == 7
+    assert subprocess.run(cmd + ["--timeout", "1", str(prog), "none"], cwd=root, timeout=60).returncode == 124
+    assert time.monotonic() - t0 < 30
+
+
 def test_world_from_environment_needs_a_launcher(monkeypatch):
     from tccl_amd import ipc
     for name in ("RANK", "WORLD_SIZE", "TCCL_RENDEZVOUS_DIR"):
