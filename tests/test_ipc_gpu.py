@@ -139,7 +139,7 @@ def test_one_shot_kernels_with_their_barriers_inside(world, tmp_path):
                 assert torch.equal(got, stacked), f"{tag} round {round_} rank {r}: all-gather"
 
 
-@pytest.mark.parametrize("world", [8, 3])
+@pytest.mark.parametrize("world", [8, 3, 2, 1])
 def test_mixed_sequence_of_kinds_and_sizes_without_host_meetings(world, tmp_path):
     """One-shot, two-shot and double-tree kernels of one workgroup per rank up to every workgroup a rank
     may hold, back to back on the same pads with the ranks out of step and no host meeting: a call with
