@@ -1,0 +1,148 @@
+"""A model of the flag protocol of the kernels that carry their barriers themselves (one launch per
+rank, the reference's blockwise_barrier, triton_barrier.py:39-142, at the start of the kernel and
+again at its end), run on the CPU under random and adversarial schedules.
+
+What the model holds: W ranks, each a stream of calls; call k of a rank has G_k workgroups (the same
+G_k in every rank), and workgroup g of a one-shot call passes two barriers with workgroup g of every
+other rank -- leading on row g, trailing on row R + g -- a two-shot call three (row R + g, row g,
+row 2 R + g).  A barrier is: store 1 into slot [row][own rank] of every peer's pad, then take
+(1 -> 0) slot [row][peer] of the own pad for every peer.  A rank's call k + 1 starts when all its
+workgroups of call k have ended.  Nothing else orders the ranks.
+
+What must hold under every schedule: no flag is ever stored over a flag that has not been taken,
+every workgroup ends (a lost flag shows as a workgroup that waits for ever), and the pads are all
+zero afterwards.  With R fixed by the pad this holds for every sequence of workgroup counts; with
+R = the call's own workgroup count -- a layout that looks equivalent -- it does not, and the model
+must say so (a model that cannot tell the two apart pins nothing)."""
+import random
+
+import pytest
+
+ONE_SHOT, TWO_SHOT = "one_shot", "two_shot"
+
+
+def rows_of(kind, g, R):
+    return (g, R + g) if kind == ONE_SHOT else (R + g, g, 2 * R + g)
+
+
+class Workgroup:
+    """Workgroup g of one rank's launch: a list of micro-steps, each one memory operation."""
+
+    def __init__(self, rank, world, rows):
+        self.steps = []
+        for row in rows:
+            for peer in range(world):
+                if peer != rank:
+                    self.steps.append(("raise", peer, row, rank))
+            for peer in range(world):
+                if peer != rank:
+                    self.steps.append(("take", rank, row, peer))
+        self.at = 0
+
+    @property
+    def done(self):
+        return self.at == len(self.steps)
+
+
+def run(world, calls, fixed_rows, seed, stall=0.0, rows=rows_of):
+    """calls: [(kind, G)], the same for every rank.  fixed_rows: R for every call, or None for R = G.
+    stall: probability per scheduling decision that the slowest rank is passed over (an adversary that
+    keeps one rank behind).  Returns (overwrites, stuck, pads_clean)."""
+    rng = random.Random(seed)
+    pads = [dict() for _ in range(world)]              # pads[owner][(row, sender)] = 0 / 1
+    at_call = [0] * world
+    live = [[] for _ in range(world)]
+
+    def launch(rank):
+        kind, G = calls[at_call[rank]]
+        R = fixed_rows if fixed_rows is not None else G
+        live[rank] = [Workgroup(rank, world, rows(kind, g, R)) for g in range(G)]
+
+    for r in range(world):
+        launch(r)
+    overwrites = 0
+    slow = rng.randrange(world)
+    while True:
+        runnable = []
+        for r in range(world):
+            if at_call[r] == len(calls):
+                continue
+            for wg in live[r]:
+                if wg.done:
+                    continue
+                op, owner, row, sender = wg.steps[wg.at]
+                if op == "raise" or pads[owner].get((row, sender), 0) == 1:
+                    runnable.append((r, wg))
+        if not runnable:
+            break
+        if stall and rng.random() < stall:
+            others = [x for x in runnable if x[0] != slow]
+            if others:
+                runnable = others
+        r, wg = rng.choice(runnable)
+        op, owner, row, sender = wg.steps[wg.at]
+        if op == "raise":
+            overwrites += pads[owner].get((row, sender), 0)
+            pads[owner][(row, sender)] = 1
+        else:
+            pads[owner][(row, sender)] = 0
+        wg.at += 1
+        if all(w.done for w in live[r]):                  # the rank's kernel has ended: its next call starts
+            at_call[r] += 1
+            if at_call[r] < len(calls):
+                launch(r)
+    stuck = any(c < len(calls) for c in at_call)
+    clean = all(v == 0 for pad in pads for v in pad.values())
+    return overwrites, stuck, clean
+
+
+def sequences(rng, kinds, length):
+    return [(rng.choice(kinds), rng.choice((1, 2, 3, 5))) for _ in range(length)]
+
+
+@pytest.mark.parametrize("kinds", [(ONE_SHOT,), (TWO_SHOT,)])
+def test_rows_fixed_by_the_pad_are_safe_for_every_sequence_of_sizes(kinds):
+    rng = random.Random(1)
+    for trial in range(150):
+        world = rng.choice((2, 3, 4))
+        calls = sequences(rng, kinds, 6)
+        for stall in (0.0, 0.9):
+            overwrites, stuck, clean = run(world, calls, fixed_rows=5, seed=trial, stall=stall)
+            assert (overwrites, stuck, clean) == (0, False, True), (world, calls, stall)
+
+
+@pytest.mark.parametrize("kinds", [(ONE_SHOT,), (TWO_SHOT,)])
+def test_the_model_catches_rows_that_move_with_the_workgroup_count(kinds):
+    """R = G: a call with more workgroups than the one before it raises leading flags on rows where a
+    slow peer still holds the last call's trailing flags."""
+    rng = random.Random(2)
+    failures = 0
+    for trial in range(150):
+        calls = sequences(rng, kinds, 6)
+        overwrites, stuck, clean = run(3, calls, fixed_rows=None, seed=trial, stall=0.9)
+        failures += bool(overwrites or stuck or not clean)
+    assert failures > 10
+    # ... and it is the growth that does it: with the same count in every call the moving layout is the fixed one
+    for trial in range(50):
+        calls = [(rng.choice(kinds), 3) for _ in range(6)]
+        assert run(3, calls, fixed_rows=None, seed=trial, stall=0.9) == (0, False, True)
+
+
+def rows_with_a_pad_per_family(kind, g, R):
+    """The one-shot family's rows beyond every row of the two-shot family: another pad."""
+    return tuple(1000 + row for row in rows_of(kind, g, R)) if kind == ONE_SHOT else rows_of(kind, g, R)
+
+
+def test_families_need_pads_of_their_own():
+    """One-shot and two-shot calls on the SAME pads, both with rows fixed by the pad: the two-shot call's
+    leading barrier sits on the rows of the one-shot call's trailing barrier, and a flag is lost.  With a
+    pad per family nothing is."""
+    rng = random.Random(3)
+    shared = separate = 0
+    for trial in range(150):
+        calls = sequences(rng, (ONE_SHOT, TWO_SHOT), 6)
+        o, s, c = run(3, calls, fixed_rows=5, seed=trial, stall=0.9)
+        shared += bool(o or s or not c)
+        o, s, c = run(3, calls, fixed_rows=5, seed=trial, stall=0.9, rows=rows_with_a_pad_per_family)
+        separate += bool(o or s or not c)
+    assert shared > 10 and separate == 0
