@@ -19,21 +19,30 @@ import random
 import pytest
 
 ONE_SHOT, TWO_SHOT = "one_shot", "two_shot"
+# the two-shot kernel without its own leading and trailing barrier (only the one between the shots, row g),
+# and the barrier as a launch of its own on pads of its own, whose sender waits for its slot to be clear
+TWO_SHOT_BARE, BARRIER_LAUNCH = "two_shot_bare", "barrier_launch"
 
 
 def rows_of(kind, g, R):
-    return (g, R + g) if kind == ONE_SHOT else (R + g, g, 2 * R + g)
+    if kind == ONE_SHOT:
+        return (g, R + g)
+    if kind == TWO_SHOT:
+        return (R + g, g, 2 * R + g)
+    if kind == TWO_SHOT_BARE:
+        return (g,)
+    return (5000 + g,)
 
 
 class Workgroup:
     """Workgroup g of one rank's launch: a list of micro-steps, each one memory operation."""
 
-    def __init__(self, rank, world, rows):
+    def __init__(self, rank, world, rows, sender_waits=False):
         self.steps = []
         for row in rows:
             for peer in range(world):
                 if peer != rank:
-                    self.steps.append(("raise", peer, row, rank))
+                    self.steps.append(("raise_when_clear" if sender_waits else "raise", peer, row, rank))
             for peer in range(world):
                 if peer != rank:
                     self.steps.append(("take", rank, row, peer))
@@ -56,7 +65,7 @@ def run(world, calls, fixed_rows, seed, stall=0.0, rows=rows_of):
     def launch(rank):
         kind, G = calls[at_call[rank]]
         R = fixed_rows if fixed_rows is not None else G
-        live[rank] = [Workgroup(rank, world, rows(kind, g, R)) for g in range(G)]
+        live[rank] = [Workgroup(rank, world, rows(kind, g, R), kind == BARRIER_LAUNCH) for g in range(G)]
 
     for r in range(world):
         launch(r)
@@ -71,7 +80,8 @@ def run(world, calls, fixed_rows, seed, stall=0.0, rows=rows_of):
                 if wg.done:
                     continue
                 op, owner, row, sender = wg.steps[wg.at]
-                if op == "raise" or pads[owner].get((row, sender), 0) == 1:
+                slot = pads[owner].get((row, sender), 0)
+                if op == "raise" or slot == (1 if op == "take" else 0):
                     runnable.append((r, wg))
         if not runnable:
             break
@@ -81,7 +91,7 @@ def run(world, calls, fixed_rows, seed, stall=0.0, rows=rows_of):
                 runnable = others
         r, wg = rng.choice(runnable)
         op, owner, row, sender = wg.steps[wg.at]
-        if op == "raise":
+        if op != "take":
             overwrites += pads[owner].get((row, sender), 0)
             pads[owner][(row, sender)] = 1
         else:
@@ -146,3 +156,25 @@ def test_families_need_pads_of_their_own():
         o, s, c = run(3, calls, fixed_rows=5, seed=trial, stall=0.9, rows=rows_with_a_pad_per_family)
         separate += bool(o or s or not c)
     assert shared > 10 and separate == 0
+
+
+def test_barrier_launches_around_the_bare_kernel_mix_with_the_kernel_that_has_its_own():
+    """The two-shot all-reduce as barrier launch + kernel + barrier launch and as one launch with the
+    barriers inside, in any order on the same kernel pads (the barrier launches have pads of their own)."""
+    rng = random.Random(4)
+    for trial in range(150):
+        calls = []
+        for _ in range(5):
+            G = rng.choice((1, 2, 3, 5))
+            if rng.random() < 0.5:
+                calls.append((TWO_SHOT, G))
+            else:
+                calls += [(BARRIER_LAUNCH, 4), (TWO_SHOT_BARE, G), (BARRIER_LAUNCH, 4)]
+        for stall in (0.0, 0.9):
+            assert run(3, calls, fixed_rows=5, seed=trial, stall=stall) == (0, False, True), calls
+    # the barrier launch's own protocol, back to back: safe because its sender waits for a clear slot ...
+    for trial in range(50):
+        assert run(3, [(BARRIER_LAUNCH, 4)] * 8, fixed_rows=5, seed=trial, stall=0.9) == (0, False, True)
+    # ... which a barrier on ONE row without that wait is not (the bare kernel's row, called back to back)
+    bad = sum(run(3, [(TWO_SHOT_BARE, 3)] * 8, fixed_rows=5, seed=trial, stall=0.9) != (0, False, True) for trial in range(50))
+    assert bad > 5
