@@ -394,7 +394,8 @@ int tccl_timeout_flag_destroy(uint32_t *flag);
 /* Buffers that several processes on one GPU can map: what the reference gets from
  * _SymmetricMemory.empty_strided_p2p (triton_one_shot_all_reduce_no_128.py:116-122) and
  * rendezvous (:82).  tccl_symm_alloc returns a zero-filled device allocation of its own (below
- * 2 GiB; it waits for the null stream, so the zeros are in place before a peer can map it); tccl_ipc_export writes its 64-byte handle, which the host side carries to the peers;
+ * 2 GiB; it waits for the null stream, so the zeros are in place before a peer can map it);
+ * tccl_ipc_export writes its 64-byte handle, which the host side carries to the peers;
  * tccl_ipc_open maps a peer's allocation into this process and returns its address here, good for
  * every pointer table of this header; tccl_ipc_close unmaps it.  These four calls allocate, map or
  * synchronise: they belong to set-up, not to the hot path. */
