@@ -85,7 +85,7 @@ class IpcWorld:
         self._allocs: List[int] = []          # own allocations
         self._opened: List[int] = []          # peers' allocations mapped here
         self._tables = {}                     # own buffer address -> (all ranks' addresses, bytes, dtype)
-        self._tree_pads = {}                  # (kernel family, pad size) -> table of all ranks' pads for kernels that signal inside a launch
+        self._family_pads = {}                  # (kernel family, pad size) -> table of all ranks' pads for kernels that signal inside a launch
         self._count = 0
         self._host_barriers = 0
         self._epoch = 0                       # resets so far: time-outs are published per epoch
@@ -213,9 +213,9 @@ class IpcWorld:
         while a slower peer has yet to take its last flags may only be followed, on the same pads, by a
         kernel that keeps those rows for the same purpose."""
         key = (family, nbytes)
-        if key not in self._tree_pads:
-            self._tree_pads[key] = _lib.ptr_array(self._exchange(self._alloc(nbytes), "kpad"))
-        return self._tree_pads[key]
+        if key not in self._family_pads:
+            self._family_pads[key] = _lib.ptr_array(self._exchange(self._alloc(nbytes), "kpad"))
+        return self._family_pads[key]
 
     def _own_launch(self, name: str, family: str, tensor: torch.Tensor, pad_bytes: int, tail_args, cfg,
                     own_barriers: bool = False) -> torch.Tensor:
@@ -427,7 +427,7 @@ class IpcWorld:
         _as_tensor(self._pad_ptrs[self.rank], self.PAD_BYTES, self.device).zero_()
         # the pads of the kernels that signal inside a launch, control words included: a wait that
         # expired there leaves flags standing that the next collective would take for its own
-        for (_, nbytes), table in self._tree_pads.items():
+        for (_, nbytes), table in self._family_pads.items():
             _as_tensor(table[self.rank], nbytes, self.device).zero_()
         torch.cuda.synchronize(self.device)
         self._flag[0] = 0
