@@ -68,7 +68,7 @@ def main() -> int:
         print(f"{'per buffer':>10s} {'barrier':>10s} | {'one-shot x3':>11s} {'fused':>11s} | {'rs x3':>10s} {'fused':>10s} | "
               f"{'ag x3':>10s} {'fused':>10s} | {'two-shot x3':>11s} {'fused':>11s} | {'tree x3':>11s} {'fused':>11s}", flush=True)
     for kib in sizes:
-        numel = kib << 9
+        numel = (kib << 9) // (8 * size) * (8 * size)      # whole 16-byte vectors per rank's share in any world
         t = world.empty(numel, torch.bfloat16)
         t.copy_(torch.randn(numel, dtype=torch.bfloat16) * 0.01)
         ptrs = _lib.ptr_array(world._tables[t.data_ptr()][0])
