@@ -94,9 +94,11 @@ class IpcWorld:
         # signal pads: one per rank, every rank maps all of them
         self._pad_ptrs = self._exchange(self._alloc(self.PAD_BYTES), "pad")
         self._pad_array = _lib.ptr_array(self._pad_ptrs)
-        # ... and the pads of the one-shot kernels that carry their barriers themselves, so that a rank's
-        # first collective never has to wait on the host for a peer that is late
+        # ... and the pads of the one-shot and two-shot kernels that carry their barriers themselves, so that
+        # a rank's first collective never has to wait on the host for a peer that is late (the double tree's
+        # pads depend on the input's size and are made when a size is first used)
         self._kernel_pads(self.ONE_SHOT_PAD_BYTES, "one_shot")
+        self._kernel_pads(self.TWO_SHOT_PAD_BYTES, "two_shot")
 
     @classmethod
     def from_env(cls, device="cuda:0", timeout_s: float = 60.0) -> "IpcWorld":
