@@ -18,7 +18,10 @@ The in-place forms rescale the buffer before every call so that values stay fini
 kernel is part of their time.  On one GPU the W processes' queues take turns, so these times say how
 the forms compare with each other here, not what they would cost with a GPU per rank.
 ``--json``: one JSON line per size instead of the table (bench.py reads those); ``--sizes``: buffer sizes
-in KiB instead of 64 KiB ... 256 MiB."""
+in KiB instead of 64 KiB ... 256 MiB.
+``--timeline``: instead of all that, 40 barrier launches per rank, each between two one-lane kernels that store
+the GPU's wall clock (benchlib/probe.hip), and rank 0 prints when every rank's stream reached each barrier and when
+it left it, on that common clock: who the others wait for, and for how long."""
 import ctypes
 import json
 import os
@@ -35,7 +38,46 @@ COLUMNS = ("barrier", "one_shot_x3", "one_shot_fused", "reduce_scatter_x3", "red
            "all_gather_fused", "two_shot_x3", "two_shot_fused", "double_tree_x3", "double_tree_fused")
 
 
+def timeline(world) -> int:
+    """When each rank's stream reaches a barrier and when it leaves it, on the GPU's one wall clock."""
+    import numpy as np
+    from benchlib import probe
+    plib = probe.load()
+    rank, size, rounds = world.rank, world.world_size, 40
+    stamps = torch.zeros(2 * rounds, dtype=torch.int64, device=world.device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(8):
+        world.barrier()
+    torch.cuda.synchronize()
+    world.host_barrier()
+    for i in range(rounds):
+        assert plib.tccl_probe_stamp(stamps.data_ptr() + 16 * i, stream) == 0
+        world.barrier()
+        assert plib.tccl_probe_stamp(stamps.data_ptr() + 16 * i + 8, stream) == 0
+    torch.cuda.synchronize()
+    world.check()
+    np.save(os.path.join(world.directory, f"timeline.rank{rank}.npy"), stamps.cpu().numpy())
+    world.host_barrier()
+    if rank == 0:
+        t = np.stack([np.load(os.path.join(world.directory, f"timeline.rank{r}.npy")) for r in range(size)]).reshape(size, rounds, 2)
+        t = (t - t[:, 8:, 0].min()) / 100.0                       # us since the first arrival of round 8
+        print(f"{size} processes, one barrier launch per rank and round; us on the GPU's wall clock, rounds 8..{rounds - 1}")
+        print("round | arrival of each rank's stream after the round's first (rank order) | all ranks left after | round lasted")
+        for i in range(8, rounds):
+            first = t[:, i, 0].min()
+            lags = " ".join(f"{v - first:6.1f}" for v in t[:, i, 0])
+            print(f"{i:5d} | {lags} | {t[:, i, 1].max() - first:6.1f} | {t[:, i, 1].max() - t[:, i - 1, 1].max():6.1f}")
+        lag = np.sort(t[:, 8:, 0] - t[:, 8:, 0].min(axis=0, keepdims=True), axis=0)     # per round, ranks by arrival
+        print("mean arrival after the round's first, k-th to arrive: " + " ".join(f"{v:.1f}" for v in lag.mean(axis=1)))
+        own = (t[:, 8:, 1] - t[:, 8:, 0]).mean(axis=1)
+        print("mean time between a rank's own two stamps (rank order): " + " ".join(f"{v:.1f}" for v in own), flush=True)
+    world.close()
+    return 0
+
+
 def main() -> int:
+    if "--timeline" in sys.argv:
+        return timeline(ipc.IpcWorld.from_env())
     as_json = "--json" in sys.argv
     sizes = (64, 1024, 4096, 16384, 65536, 262144)
     if "--sizes" in sys.argv:

@@ -35,6 +35,9 @@ int tccl_probe_copy(const void *src, void *dst, size_t bytes, void *stream);
 int tccl_probe_sum_timed(const void *const *bufs, void *out, size_t bytes_per_buffer, long long *stamps, void *stream);
 /* One empty kernel: what a timed single launch costs when the kernel does nothing. */
 int tccl_probe_empty(void *stream);
+/* A one-lane kernel that stores the GPU's 100 MHz wall clock at `slot` (device memory): where a
+ * stream has got to, on a clock that all processes sharing the GPU read alike. */
+int tccl_probe_stamp(long long *slot, void *stream);
 /* An empty kernel of `workgroups` x 256 lanes, and the same grid with every lane loading one
  * 16-byte vector from src and storing it to dst (both workgroups x 4 KiB): what a short
  * streaming kernel costs whatever it moves. */

@@ -280,6 +280,12 @@ __global__ void __launch_bounds__(kPhasedBlock) probe_sum_timed_kernel(ProbeSrc<
 
 __global__ void probe_empty_kernel() {}
 
+// One lane writes the 100 MHz wall clock, which every process on the GPU reads the same.
+__global__ void probe_stamp_kernel(long long *slot)
+{
+    if (threadIdx.x == 0) *slot = static_cast<long long>(wall_clock64());
+}
+
 // The same grid as a sum launch doing nothing, and doing the least a streaming kernel can do:
 // every lane loads one vector and stores it (one round trip to memory each way).  Their
 // durations are the part of a short kernel's time that does not depend on its bytes.
@@ -375,6 +381,13 @@ extern "C" int tccl_probe_sum_timed(const void *const *bufs, void *out, size_t b
 extern "C" int tccl_probe_empty(void *stream)
 {
     hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream));
+    return hip_code(hipGetLastError());
+}
+
+extern "C" int tccl_probe_stamp(long long *slot, void *stream)
+{
+    if (slot == nullptr) return TCCL_EINVAL;
+    hipLaunchKernelGGL(probe_stamp_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), slot);
     return hip_code(hipGetLastError());
 }
 

@@ -19,6 +19,7 @@ SIGNATURES = {
     "tccl_probe_copy": (_I, [_P, _P, _SZ, _P]),
     "tccl_probe_sum_timed": (_I, [_PP, _P, _SZ, _P, _P]),
     "tccl_probe_empty": (_I, [_P]),
+    "tccl_probe_stamp": (_I, [_P, _P]),
     "tccl_probe_empty_grid": (_I, [_I, _P]),
     "tccl_probe_touch": (_I, [_P, _P, _I, _P]),
     "tccl_probe_placement": (_I, [_P, _I, _I, _P]),

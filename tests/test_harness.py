@@ -84,3 +84,21 @@ def test_sweep_with_a_process_per_rank(op):
     recs = [r for r in recs if r is not None]
     assert [r[1] for r in recs] == [2 * ((1 << 20) >> i) for i in range(10)], proc.stdout
     assert all(r[0] == "tccl_amd" and 0 < r[2] < float("inf") for r in recs)
+
+
+@pytest.mark.gpu
+def test_barrier_timeline_with_a_process_per_rank():
+    """``benchlib/ipc_forms.py --timeline`` with 3 processes: every rank stamps the GPU's wall clock before and
+    after each barrier launch; the table rank 0 prints has a line per round with one arrival per rank, the
+    first of them 0, and every rank leaves a barrier after the last has arrived."""
+    cmd = [sys.executable, "-m", "tccl_amd.launch", "--nproc-per-node", "3", os.path.join(ROOT, "benchlib", "ipc_forms.py"),
+           "--timeline"]
+    proc = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=150)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    rows = [ln.split("|") for ln in proc.stdout.splitlines() if ln[:6].strip().isdigit()]
+    assert len(rows) == 32, proc.stdout
+    for _, arrivals, left, lasted in rows:
+        arrivals = [float(v) for v in arrivals.split()]
+        assert len(arrivals) == 3 and min(arrivals) == 0.0
+        assert float(left) >= max(arrivals) and 0 < float(lasted) < 1e5
+    assert "mean arrival after the round's first" in proc.stdout
