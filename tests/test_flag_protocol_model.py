@@ -13,7 +13,13 @@ What must hold under every schedule: no flag is ever stored over a flag that has
 every workgroup ends (a lost flag shows as a workgroup that waits for ever), and the pads are all
 zero afterwards.  With R fixed by the pad this holds for every sequence of workgroup counts; with
 R = the call's own workgroup count -- a layout that looks equivalent -- it does not, and the model
-must say so (a model that cannot tell the two apart pins nothing)."""
+must say so (a model that cannot tell the two apart pins nothing).
+
+The pipelined double tree (triton_double_tree_allreduce.py:254-335 as designed: wait for the children's
+chunk, reduce, signal the parent; wait for the parent's result, copy, signal the children) is modelled
+the same way, chunk flags and barriers together: with its own leading and trailing barrier, or between
+two barrier launches, every sequence of chunk counts, workgroup counts and lags ends with clean pads;
+without a barrier after it a slow leaf loses a flag, and the model says so."""
 import random
 
 import pytest
@@ -34,23 +40,32 @@ def rows_of(kind, g, R):
     return (5000 + g,)
 
 
-class Workgroup:
-    """Workgroup g of one rank's launch: a list of micro-steps, each one memory operation."""
+def barrier_steps(rank, world, row, sender_waits=False):
+    """One blockwise barrier of a workgroup on `row`: raise the own slot in every peer's pad, take every
+    peer's slot in the own pad."""
+    steps = [("raise_when_clear" if sender_waits else "raise", peer, row, rank) for peer in range(world) if peer != rank]
+    return steps + [("take", rank, row, peer) for peer in range(world) if peer != rank]
 
-    def __init__(self, rank, world, rows, sender_waits=False):
-        self.steps = []
-        for row in rows:
-            for peer in range(world):
-                if peer != rank:
-                    self.steps.append(("raise_when_clear" if sender_waits else "raise", peer, row, rank))
-            for peer in range(world):
-                if peer != rank:
-                    self.steps.append(("take", rank, row, peer))
+
+class Workgroup:
+    """Workgroup g of one rank's launch: a list of micro-steps, each one memory operation
+    (op, owner of the pad, slot key, sender)."""
+
+    def __init__(self, steps):
+        self.steps = steps
         self.at = 0
 
     @property
     def done(self):
         return self.at == len(self.steps)
+
+
+def workgroups_of(kind, rank, world, G, R, rows):
+    """The workgroups of one rank's launch of a call (kind, G)."""
+    if isinstance(kind, tuple):                          # ("tree", chunks of tree a, chunks of tree b, lag, own barriers)
+        return tree_workgroups(kind, rank, world, G)
+    return [Workgroup([st for row in rows(kind, g, R) for st in barrier_steps(rank, world, row, kind == BARRIER_LAUNCH)])
+            for g in range(G)]
 
 
 def run(world, calls, fixed_rows, seed, stall=0.0, rows=rows_of):
@@ -65,7 +80,7 @@ def run(world, calls, fixed_rows, seed, stall=0.0, rows=rows_of):
     def launch(rank):
         kind, G = calls[at_call[rank]]
         R = fixed_rows if fixed_rows is not None else G
-        live[rank] = [Workgroup(rank, world, rows(kind, g, R), kind == BARRIER_LAUNCH) for g in range(G)]
+        live[rank] = workgroups_of(kind, rank, world, G, R, rows)
 
     for r in range(world):
         launch(r)
@@ -178,3 +193,92 @@ def test_barrier_launches_around_the_bare_kernel_mix_with_the_kernel_that_has_it
     # ... which a barrier on ONE row without that wait is not (the bare kernel's row, called back to back)
     bad = sum(run(3, [(TWO_SHOT_BARE, 3)] * 8, fixed_rows=5, seed=trial, stall=0.9) != (0, False, True) for trial in range(50))
     assert bad > 5
+
+
+# ------------------------------------------------------------------ the pipelined double tree, one launch per rank
+TREE_BARRIER_ROWS = 512                  # the barriers' second block of rows starts here, whatever G is
+
+
+def tree_tables(world):
+    """(parent, child0, child1) and height per tree and rank, as the kernel holds them; height 0 = leaf,
+    the extra node on top (one child, tree.py:133-136) has the largest."""
+    import tccl_amd
+    nbr = [[None] * world for _ in range(2)]
+    for r in range(world):
+        six = tccl_amd.get_parents_and_children(world, r)
+        nbr[0][r], nbr[1][r] = tuple(six[:3]), tuple(six[3:])
+    height = [[0] * world for _ in range(2)]
+
+    def h(t, r):
+        kids = [c for c in nbr[t][r][1:] if c >= 0]
+        return 0 if not kids else 1 + max(h(t, c) for c in kids)
+    for t in range(2):
+        for r in range(world):
+            height[t][r] = h(t, r)
+    return nbr, height
+
+
+def tree_workgroups(kind, rank, world, G):
+    """tree_pipelined_walk: workgroup g takes chunks g, g + G, ... of both trees; in round i the up-sweep
+    step of its i-th chunk and the down-sweep step of its (i - lag)-th; with own barriers a blockwise
+    barrier before and after (rows g and 512 + g of the barriers' block)."""
+    _, nchunks_a, nchunks_b, lag, own_barriers = kind
+    nchunks = (nchunks_a, nchunks_b)
+    nbr, height = tree_tables(world)
+    top = max(height[0])
+    most = max(nchunks)
+    out = []
+    for g in range(min(G, most)):                       # workgroups beyond the last chunk leave at once
+        steps = []
+        if own_barriers:
+            steps += barrier_steps(rank, world, ("bar", g))
+        rounds = (most - g + G - 1) // G
+        for i in range(rounds + lag):
+            if i < rounds:
+                c = g + i * G
+                for t in range(2):
+                    parent, c0, c1 = nbr[t][rank]
+                    if c >= nchunks[t] or height[t][rank] == 0:
+                        continue
+                    steps += [("take", rank, ("chunk", t, c), kid) for kid in (c0, c1) if kid >= 0 and height[t][kid] > 0]
+                    to = parent if height[t][rank] != top else c0
+                    steps.append(("raise", to, ("chunk", t, c), rank))
+            if i >= lag:
+                c = g + (i - lag) * G
+                for t in range(2):
+                    parent, c0, c1 = nbr[t][rank]
+                    if c >= nchunks[t] or height[t][rank] == top:
+                        continue
+                    steps.append(("take", rank, ("chunk", t, c), parent))
+                    steps += [("raise", kid, ("chunk", t, c), rank) for kid in (c0, c1) if kid >= 0]
+        if own_barriers:
+            steps += barrier_steps(rank, world, ("bar", TREE_BARRIER_ROWS + g))
+        out.append(Workgroup(steps))
+    return out
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_double_tree_with_its_own_barriers_is_safe_for_every_sequence_of_sizes_and_grids(world):
+    """Calls of different chunk counts, workgroup counts and lags back to back on the same pads: every
+    workgroup ends (nothing waits in a circle), no flag is stored over one not yet taken, pads end clean."""
+    rng = random.Random(5)
+    for trial in range(40):
+        calls = [(("tree", rng.choice((1, 2, 5, 9)), rng.choice((1, 3, 5, 8)), rng.choice((0, 1, 3)), True), rng.choice((1, 2, 3, 6)))
+                 for _ in range(4)]
+        for stall in (0.0, 0.9):
+            assert run(world, calls, fixed_rows=5, seed=trial, stall=stall) == (0, False, True), calls
+
+
+def test_double_tree_without_a_barrier_after_it_loses_a_leaf_s_flag():
+    """What the trailing barrier is for: a parent does not wait for a leaf child before it sends the next
+    call's result down, so without a barrier between two calls a slow leaf still holds the last call's flag
+    in that slot.  A barrier launch either side of the bare kernel is the other safe form."""
+    rng = random.Random(6)
+    bare = ("tree", 3, 3, 1, False)
+    bad = sum(run(4, [(bare, 2)] * 4, fixed_rows=5, seed=trial, stall=0.9) != (0, False, True) for trial in range(60))
+    assert bad > 5
+    for trial in range(40):
+        calls = []
+        for _ in range(3):
+            calls += [(BARRIER_LAUNCH, 4), (("tree", rng.choice((1, 3, 6)), 3, 1, False), rng.choice((1, 2, 4))), (BARRIER_LAUNCH, 4)]
+        assert run(4, calls, fixed_rows=5, seed=trial, stall=0.9) == (0, False, True), calls
