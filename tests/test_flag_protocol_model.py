@@ -282,3 +282,63 @@ def test_double_tree_without_a_barrier_after_it_loses_a_leaf_s_flag():
         for _ in range(3):
             calls += [(BARRIER_LAUNCH, 4), (("tree", rng.choice((1, 3, 6)), 3, 1, False), rng.choice((1, 2, 4))), (BARRIER_LAUNCH, 4)]
         assert run(4, calls, fixed_rows=5, seed=trial, stall=0.9) == (0, False, True), calls
+
+
+# ------------------------------------------------------------------ one launch for all ranks: which workgroup takes which place
+def run_one_launch(world, G, resident, lists, draw, seed):
+    """All W ranks' workgroups in ONE launch of world * G workgroups of which at most `resident` run at a
+    time, started in hardware order as slots come free (a workgroup holds its slot until it ends).  Place
+    (rank, g) meets the places with the same g in a blockwise barrier (the two-shot kernel between its
+    shots).  By hardware index workgroup b is place (b // G, b % G); drawn (take_place), a workgroup that
+    starts on XCD x takes the next place of list x -- the places with g % lists == x in the order (g, rank) --
+    or of the following lists when that one is used up.  Returns True when every workgroup has ended."""
+    rng = random.Random(seed)
+    total = world * G
+    order = [[(g, r) for g in range(G) if g % lists == x for r in range(world)] for x in range(lists)]
+    drawn = [0] * lists
+    pads = [dict() for _ in range(world)]
+    running, started, ended = [], 0, 0
+    while ended < total:
+        while started < total and len(running) < resident:
+            if draw:
+                x = rng.randrange(lists)                              # whichever XCD the hardware picked
+                while drawn[x] == len(order[x]):
+                    x = (x + 1) % lists
+                g, rank = order[x][drawn[x]]
+                drawn[x] += 1
+            else:
+                rank, g = started // G, started % G
+            running.append(Workgroup(barrier_steps(rank, world, g)))
+            started += 1
+        runnable = []
+        for wg in running:
+            op, owner, row, sender = wg.steps[wg.at]
+            if op == "raise" or pads[owner].get((row, sender), 0) == 1:
+                runnable.append(wg)
+        if not runnable:
+            return False                                              # everything resident waits for a place not yet started
+        wg = rng.choice(runnable)
+        op, owner, row, sender = wg.steps[wg.at]
+        pads[owner][(row, sender)] = 1 if op == "raise" else 0
+        wg.at += 1
+        if wg.done:
+            running.remove(wg)
+            ended += 1
+    return True
+
+
+def test_drawn_places_make_progress_whatever_is_resident():
+    """With places drawn in the order in which workgroups really start, at most lists * (W - 1) workgroups can
+    be waiting for a member of their group that has not started, so any residency above that drains any grid;
+    with places bound to the hardware index the whole grid must be resident."""
+    rng = random.Random(7)
+    for trial in range(200):
+        world, lists = rng.choice((2, 3, 4)), rng.choice((1, 2, 4))
+        G = rng.choice((1, 3, 8, 17))
+        resident = lists * (world - 1) + 1 + rng.choice((0, 1, 5))
+        assert run_one_launch(world, G, resident, lists, True, trial), (world, G, resident, lists)
+    # by index: fine when everything is resident, stuck as soon as a rank's workgroups fill the slots
+    assert all(run_one_launch(3, 8, 24, 2, False, trial) for trial in range(20))
+    assert not any(run_one_launch(3, 8, 8, 2, False, trial) for trial in range(20))
+    # ... and the bound is tight: one slot fewer than lists * (W - 1) + 1 can be filled with waiting workgroups
+    assert not all(run_one_launch(3, 8, 4, 2, True, trial) for trial in range(200))
